@@ -1,0 +1,231 @@
+#!/usr/bin/env python3
+"""Benchmark of the LBI bounded-interface backward hot path on one MI355X.
+
+One "step" is one pass of the interface suffix scan at the scale configuration
+(B=64 batch elements, K=128 regions, d=256 interface width, fp32): all K suffix
+matrices (``lbi_suffix_scan``) plus all K suffix cotangents
+(``lbi_suffix_cotangents``), inputs resident in HBM.  ``value`` is composed
+pullbacks per second, ``B*K / t_step``.
+
+Prints ONE JSON line.  Besides the contract keys it carries
+
+* ``roofline``      - the dominant kernel (the d x d suffix-product kernel) against the
+                      MI355X fp32-MFMA peak, from HIP-event timing of that kernel alone;
+* ``cpu_baseline``  - the reference's CPU algorithm (log-depth torch scan) timed on the
+                      host cores of the same box on a bounded batch slice;
+* ``extra``         - the other measured variants (bf16 storage, cotangent-only chain,
+                      attention input-pullback) with their own roofline figures.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16/fp16 matrix peak
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
+
+SCAN_B, SCAN_K, SCAN_D = 64, 128, 256
+
+
+def _parse() -> argparse.Namespace:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline scan (used for profiling)")
+    ap.add_argument("--cpu-sample-batch", type=int, default=8)
+    return ap.parse_args()
+
+
+def _time_events(fn, steps: int, warmup: int):
+    """Per-call milliseconds from HIP events on the current torch stream (which is
+    the stream every kernel of this library is launched on)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(steps):
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        stop.record()
+        stop.synchronize()
+        times.append(float(start.elapsed_time(stop)))
+    return times
+
+
+def _scan_inputs(device, dtype):
+    import torch
+
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    noise = torch.randn(SCAN_B, SCAN_K, SCAN_D, SCAN_D, generator=gen, dtype=torch.float32)
+    mats = torch.eye(SCAN_D, dtype=torch.float32) + noise * (0.01 / SCAN_D) ** 0.5
+    g = torch.randn(SCAN_B, SCAN_D, generator=gen, dtype=torch.float32)
+    return mats.to(dtype).to(device), g.to(device)
+
+
+def _cpu_baseline(sample_batch: int) -> dict:
+    """The reference's CPU path (log-depth torch scan) on `sample_batch` batch elements."""
+    import torch
+
+    from oracle import scan as oscan
+
+    mats, g = oscan.make_scan_inputs(sample_batch, SCAN_K, SCAN_D, kind="near_identity", seed=0)
+    oscan.suffix_scan_levels(mats[:1, :8])  # warm the BLAS threads
+    t0 = time.perf_counter()
+    suffix = oscan.suffix_scan_levels(mats)
+    oscan.suffix_cotangents_from_matrices(suffix[:, :SCAN_K], g)
+    dt = time.perf_counter() - t0
+    return {
+        "value": sample_batch * SCAN_K / dt,
+        "unit": "composed_pullbacks/s",
+        "cores": int(torch.get_num_threads()),
+        "kind": "port",
+        "sample": f"B={sample_batch} of {SCAN_B} batch elements, K={SCAN_K}, d={SCAN_D}, fp32, "
+                  f"log-depth torch scan + mat-vecs, {dt:.2f} s wall",
+    }
+
+
+def main() -> int:
+    args = _parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the path has no cross-GPU "
+              "dependency; shard the batch and run one process per GPU); rerun with --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    from latent_bounded_interfaces_amd import _lib
+
+    lib = _lib.load()
+    stream = _lib.current_stream_ptr(device)
+
+    def scan_call(mats, out):
+        _lib.check(lib.lbi_suffix_scan(mats.data_ptr(), out.data_ptr(), SCAN_B, SCAN_K, SCAN_D,
+                                       _lib.dtype_code(mats.dtype), _lib.LBI_F32, stream), "lbi_suffix_scan")
+
+    def cot_call(mats, g, out):
+        _lib.check(lib.lbi_suffix_cotangents(mats.data_ptr(), g.data_ptr(), out.data_ptr(), SCAN_B, SCAN_K,
+                                             SCAN_D, _lib.dtype_code(mats.dtype), stream),
+                   "lbi_suffix_cotangents")
+
+    mats, g = _scan_inputs(device, torch.float32)
+    out = torch.empty((SCAN_B, SCAN_K + 1, SCAN_D, SCAN_D), device=device, dtype=torch.float32)
+    cot = torch.empty((SCAN_B, SCAN_K + 1, SCAN_D), device=device, dtype=torch.float32)
+
+    def step():
+        scan_call(mats, out)
+        cot_call(mats, g, cot)
+
+    # ---- headline: exactly `steps` timed steps between synchronisations ----------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = SCAN_B * SCAN_K / (wall / args.steps)
+
+    # ---- dominant kernel alone, HIP events on its stream ------------------------------
+    scan_ms = _time_events(lambda: scan_call(mats, out), args.steps, 2)
+    scan_avg = statistics.fmean(scan_ms)
+    scan_flops = SCAN_B * (SCAN_K - 1) * 2 * SCAN_D ** 3
+    scan_bytes = SCAN_B * SCAN_K * SCAN_D * SCAN_D * (4 + 4)
+    achieved_tflops = scan_flops / (scan_avg * 1e-3) / 1e12
+    first = out.clone()
+    scan_call(mats, out)
+    torch.cuda.synchronize()
+    bit_stable = bool(torch.equal(first, out))
+    del first
+
+    result = {
+        "metric": "scan composed-pullbacks/s + attn-pullback TFLOP/s, % of MI355X roofline",
+        "value": value,
+        "unit": "composed_pullbacks/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "interface suffix scan B=64 K=128 d=256 fp32: all K suffix matrices + all K cotangents",
+            "B": SCAN_B, "K": SCAN_K, "d": SCAN_D,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "scan_mfma_kernel<float,256,...> (lbi_suffix_scan)",
+            "achieved": achieved_tflops,
+            "peak": PEAK_FP32_MFMA_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved_tflops / PEAK_FP32_MFMA_TFLOPS,
+            "traffic": None,
+            "kernel_ms_avg": scan_avg,
+            "kernel_ms_min": min(scan_ms),
+            "algorithmic_flops": scan_flops,
+            "algorithmic_bytes": scan_bytes,
+            "hbm_gbs": scan_bytes / (scan_avg * 1e-3) / 1e9,
+        },
+        "bit_stable_rerun": bit_stable,
+    }
+
+    if not args.no_extra:
+        extra = {}
+        cot_ms = _time_events(lambda: cot_call(mats, g, cot), args.steps, 2)
+        cot_avg = statistics.fmean(cot_ms)
+        cot_bytes = SCAN_B * SCAN_K * SCAN_D * SCAN_D * 4
+        extra["scan_cotangent_only_fp32"] = {
+            "kernel_ms_avg": cot_avg, "pullbacks_per_s": SCAN_B * SCAN_K / (cot_avg * 1e-3),
+            "roofline": {"bound": "hbm", "achieved": cot_bytes / (cot_avg * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": cot_bytes / (cot_avg * 1e-3) / 1e9 / PEAK_HBM_GBS},
+        }
+        mats_bf16 = mats.to(torch.bfloat16)
+        bf_ms = _time_events(lambda: scan_call(mats_bf16, out), args.steps, 2)
+        bf_avg = statistics.fmean(bf_ms)
+        bf_bytes = SCAN_B * SCAN_K * SCAN_D * SCAN_D * (2 + 4)
+        extra["scan_bf16_storage_fp32_accumulate"] = {
+            "kernel_ms_avg": bf_avg, "pullbacks_per_s": SCAN_B * SCAN_K / (bf_avg * 1e-3),
+            "tflops": scan_flops / (bf_avg * 1e-3) / 1e12,
+            "roofline": {"bound": "hbm", "achieved": bf_bytes / (bf_avg * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": bf_bytes / (bf_avg * 1e-3) / 1e9 / PEAK_HBM_GBS},
+        }
+        del mats_bf16
+        try:
+            from latent_bounded_interfaces_amd import benchmarks as lbi_bench
+
+            extra.update(lbi_bench.attention_section(steps=max(3, args.steps // 4)))
+        except ImportError:
+            pass
+        result["extra"] = extra
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = _cpu_baseline(args.cpu_sample_batch)
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,147 @@
+"""State-adjoint propagation through the interface chain, on the HIP scan kernels.
+
+Counterpart of reference backward/suffix_scan.py with the same function names,
+arguments, results and exceptions.  ``Jt[b, i, j] = d s_out[j] / d s_in[i]`` and
+``g_in = Jt @ g_out`` (reference backward/pullbacks.py:53-64).
+"""
+from __future__ import annotations
+
+from collections.abc import Sequence
+
+import torch
+
+from ..hip.interface import suffix_scan_cotangents
+from ..hip.interface import suffix_scan_pullbacks as suffix_scan_jacobian_t
+
+
+def compose_suffix_jacobian_t(state_jacobians_t: Sequence[torch.Tensor]) -> list[torch.Tensor]:
+    """All suffix products of the K matrices plus the identity, as K+1 tensors ``[B, d, d]``.
+
+    Same contract as reference backward/suffix_scan.py:10-21.
+    """
+    count = len(state_jacobians_t)
+    if count == 0:
+        return []
+    bsz, rank, rank2 = state_jacobians_t[0].shape
+    if rank != rank2:
+        raise ValueError("interface state Jacobian-transpose tensors must be square.")
+    stacked = torch.stack(list(state_jacobians_t), dim=1).contiguous()
+    suffix = suffix_scan_jacobian_t(stacked)
+    if suffix.shape != (bsz, count + 1, rank, rank):
+        raise ValueError("suffix scan returned an unexpected shape")
+    return [suffix[:, region_index].contiguous() for region_index in range(count + 1)]
+
+
+def apply_jacobian_t(
+    jacobian_t: torch.Tensor,
+    cotangent: torch.Tensor,
+    *,
+    out_dtype: torch.dtype | None = None,
+) -> torch.Tensor:
+    """``result[b] = jacobian_t[b] @ cotangent[b]`` (reference backward/suffix_scan.py:24-38).
+
+    Runs as a one-step cotangent chain on the device; accumulation is fp32 and the
+    result is cast to ``out_dtype`` (default: the cotangent's dtype).
+    """
+    if jacobian_t.dim() != 3 or cotangent.dim() != 2:
+        raise ValueError("jacobian_t must be [B, d, d] and cotangent [B, d]")
+    if out_dtype is None:
+        out_dtype = cotangent.dtype
+    chain = suffix_scan_cotangents(jacobian_t.unsqueeze(1), cotangent.to(device=jacobian_t.device))
+    return chain[:, 0].to(device=cotangent.device, dtype=out_dtype)
+
+
+def _stack_for_chain(state_jacobians_t: Sequence[torch.Tensor]) -> torch.Tensor:
+    bsz, rank, rank2 = state_jacobians_t[0].shape
+    if rank != rank2:
+        raise ValueError("interface state Jacobian-transpose tensors must be square.")
+    return torch.stack(list(state_jacobians_t), dim=1).contiguous()
+
+
+def propagate_state_adjoint_with_jacobian_scan(
+    state_jacobians_t: Sequence[torch.Tensor],
+    g_top_state: torch.Tensor,
+    *,
+    materialize_suffix: bool = False,
+) -> list[torch.Tensor]:
+    """K+1 state cotangents ``[suffix[r] @ g for r < K] + [g]``.
+
+    Same results as reference backward/suffix_scan.py:41-56.  By default the
+    cotangent-only kernel is used (one pass over the matrices, no ``d x d``
+    product); ``materialize_suffix=True`` forms the suffix matrices first, as the
+    reference does.
+    """
+    count = len(state_jacobians_t)
+    if count == 0:
+        # The reference reaches its length check with an empty suffix list here.
+        raise ValueError("suffix length mismatch.")
+    if materialize_suffix:
+        suffix = compose_suffix_jacobian_t(state_jacobians_t)
+        if len(suffix) != count + 1:
+            raise ValueError("suffix length mismatch.")
+        g_top_state = g_top_state.to(device=suffix[0].device, dtype=suffix[0].dtype)
+        g_states = [
+            apply_jacobian_t(suffix[region_index], g_top_state, out_dtype=g_top_state.dtype)
+            for region_index in range(count)
+        ]
+        g_states.append(g_top_state)
+        return g_states
+    stacked = _stack_for_chain(state_jacobians_t)
+    chain = suffix_scan_cotangents(stacked, g_top_state)
+    return [chain[:, region_index] for region_index in range(count + 1)]
+
+
+def propagate_state_adjoint_from_last_region_input(
+    state_jacobians_t: Sequence[torch.Tensor],
+    g_last_input_state: torch.Tensor,
+    *,
+    num_regions: int,
+    materialize_suffix: bool = False,
+) -> list[torch.Tensor]:
+    """Cotangents of every region's input state given the one of the last region's input.
+
+    Same contract as reference backward/suffix_scan.py:59-79: the last matrix is
+    dropped (the last region's output state never reaches the loss), length
+    mismatch raises ``ValueError``, ``num_regions`` 0 / 1 return ``[]`` / ``[g]``.
+    """
+    if len(state_jacobians_t) != num_regions:
+        raise ValueError("state_jacobians_t length mismatch.")
+    if num_regions == 0:
+        return []
+    if num_regions == 1:
+        return [g_last_input_state]
+    return propagate_state_adjoint_with_jacobian_scan(
+        state_jacobians_t[:-1], g_last_input_state, materialize_suffix=materialize_suffix
+    )
+
+
+def interface_state_jacobian_t_stats(
+    state_jacobians_t: Sequence[torch.Tensor],
+    *,
+    include_suffix: bool,
+) -> dict[str, float]:
+    """Frobenius / spectral norm diagnostics (reference backward/suffix_scan.py:105-134)."""
+    if not state_jacobians_t:
+        return {}
+    with torch.no_grad():
+        dense = torch.stack([jt.detach().float() for jt in state_jacobians_t], dim=1)
+        frob = torch.linalg.matrix_norm(dense, ord="fro", dim=(-2, -1))
+        spec = torch.linalg.matrix_norm(dense, ord=2, dim=(-2, -1))
+        rank = max(1, int(dense.shape[-1]))
+        stats = {
+            "jac_local_spec_mean": float(spec.mean().item()),
+            "jac_local_spec_max": float(spec.max().item()),
+            "jac_local_frob_mean": float(frob.mean().item()),
+            "jac_local_frob_max": float(frob.max().item()),
+            "jac_local_frob_normed_mean": float((frob / (rank ** 0.5)).mean().item()),
+        }
+        if include_suffix:
+            suffix = suffix_scan_jacobian_t(dense.contiguous())
+            suffix_spec = torch.linalg.matrix_norm(suffix, ord=2, dim=(-2, -1))
+            stats.update(
+                {
+                    "jac_suffix_spec_mean": float(suffix_spec.mean().item()),
+                    "jac_suffix_spec_max": float(suffix_spec.max().item()),
+                }
+            )
+        return stats

@@ -1,0 +1,65 @@
+// Shared host/device helpers for the gfx950 kernels of liblbi_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lbi_hip.h"
+
+namespace lbi {
+
+// Records a printf-style message for lbi_last_error() on the calling thread and
+// returns `status`, so failing paths read `return fail(LBI_ERR_INVALID, "...")`.
+int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+inline size_t dtype_size(int dtype) {
+    return dtype == LBI_F32 ? 4 : (dtype == LBI_F16 || dtype == LBI_BF16) ? 2 : 0;
+}
+
+#define LBI_HIP_CHECK(expr)                                                              \
+    do {                                                                                 \
+        hipError_t lbi_e_ = (expr);                                                      \
+        if (lbi_e_ != hipSuccess)                                                        \
+            return ::lbi::fail(LBI_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(lbi_e_)); \
+    } while (0)
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+
+// Storage element types. bf16 is carried as raw 16-bit words and widened by a
+// shift, which is exact.
+struct bf16_raw { unsigned short bits; };
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(_Float16 x) { return (float)x; }
+__device__ __forceinline__ float to_f32(bf16_raw x) { return __uint_as_float(((unsigned)x.bits) << 16); }
+
+// Round-to-nearest-even narrowing, NaN preserved as quiet NaN.
+__device__ __forceinline__ unsigned short f32_to_bf16_bits(float x) {
+    unsigned u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+
+// Four consecutive storage elements widened to fp32 with one vector load.
+// `p` must be aligned to 4 elements.
+__device__ __forceinline__ f32x4 load4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 load4(const _Float16* p) {
+    f16x4 h = *reinterpret_cast<const f16x4*>(p);
+    return f32x4{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+}
+__device__ __forceinline__ f32x4 load4(const bf16_raw* p) {
+    u16x4 h = *reinterpret_cast<const u16x4*>(p);
+    return f32x4{__uint_as_float(((unsigned)h[0]) << 16), __uint_as_float(((unsigned)h[1]) << 16),
+                 __uint_as_float(((unsigned)h[2]) << 16), __uint_as_float(((unsigned)h[3]) << 16)};
+}
+
+}  // namespace lbi

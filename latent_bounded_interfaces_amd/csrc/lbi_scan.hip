@@ -1,0 +1,404 @@
+// Suffix scan of interface pullback matrices for gfx950 (MI355X).
+//
+//   out[b, r] = mats[b, r] @ out[b, r+1],  out[b, K] = I          (matrices)
+//   out[b, r] = mats[b, r] @ out[b, r+1],  out[b, K] = g[b]       (cotangents)
+//
+// The product is a LEFT multiplication, so column blocks of the running suffix
+// are independent: a workgroup owns `CB` columns of one batch element, keeps
+// that d x CB block on chip, streams mats[b, K-1] ... mats[b, 0] from HBM once
+// and writes every suffix block as it goes.  This does K-1 products per batch
+// element (the log-depth scan of the reference, cuda/interface/suffix_scan.cu:89-108,
+// does sum_l (K - 2^l)), needs no synchronisation between workgroups, and sums
+// in a fixed order, so reruns are bit-identical.
+#include "lbi_common.h"
+
+namespace lbi {
+namespace {
+
+// ---------------------------------------------------------------------------------------
+// MFMA path: d in {32, 64, 128, 256}.
+//
+// One wave computes an RT x CB tile of the new suffix block with
+// v_mfma_f32_32x32x2_f32.  Operand layout of that instruction (lane = 32*h + m):
+//   A (32 x 2):  lane holds A[m][h]        B (2 x 32):  lane holds B[h][m]
+//   C (32 x 32): register i of the lane holds C[8*(i/4) + 4*h + i%4][m]
+// Which actual k index feeds slot h of which instruction is free as long as A and
+// B agree, so a lane loads 16 CONSECUTIVE k of its row (64 bytes; the h=0 and h=1
+// lanes of a row together cover one 128-byte line) and uses them for 16
+// instructions.  The matching B values, S[k][col] for 16 consecutive k and the
+// lane's column, are contiguous because the block is kept TRANSPOSED in LDS
+// (St[col][k], row pitch D+4 floats so 16-byte reads of 16 lanes hit 64 distinct
+// banks).  The C layout gives each lane 4 consecutive rows of one column, which is
+// one 16-byte write into St for the next step.
+//
+// A rows are private to a wave, so mats go global -> registers directly,
+// prefetched one 32-wide k chunk ahead, across step boundaries too (mats do not
+// depend on the running product).  St is double buffered: one barrier per step.
+// ---------------------------------------------------------------------------------------
+template <typename Tin, int D, int RT, int CB>
+__global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
+    const Tin* __restrict__ mats, float* __restrict__ out, int B, int K) {
+    constexpr int NW = D / RT;          // waves per workgroup
+    constexpr int NT = 64 * NW;         // threads
+    constexpr int RTILES = RT / 32;
+    constexpr int CTILES = CB / 32;
+    constexpr int NB = D / CB;          // column blocks per batch element
+    constexpr int PITCH = D + 4;
+    constexpr int NCH = D / 32;         // k chunks per step
+
+    extern __shared__ __align__(16) float lds[];  // [2][CB][PITCH]
+
+    // Workgroups are dealt round-robin to the 8 XCDs; all column blocks of one
+    // batch element get ids that are equal mod 8 so they share one L2.
+    const int id = blockIdx.x;
+    const int slot = id >> 3;
+    const int b = (slot / NB) * 8 + (id & 7);
+    const int c0 = (slot % NB) * CB;
+    if (b >= B) return;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int m = lane & 31;
+    const int h = lane >> 5;
+    const int row0 = wave * RT;
+
+    const Tin* mats_b = mats + (size_t)b * K * D * D;
+    float* out_b = out + (size_t)b * (K + 1) * D * D;
+
+    // Identity tail and the first suffix (= mats[K-1]); fill St buffer 0.
+    {
+        const Tin* a_last = mats_b + (size_t)(K - 1) * D * D;
+        float* o_last = out_b + (size_t)(K - 1) * D * D;
+        float* o_eye = out_b + (size_t)K * D * D;
+        for (int idx = tid; idx < D * CB; idx += NT) {
+            const int row = idx / CB;
+            const int col = idx % CB;
+            const float val = to_f32(a_last[row * D + c0 + col]);
+            o_last[row * D + c0 + col] = val;
+            o_eye[row * D + c0 + col] = (row == c0 + col) ? 1.0f : 0.0f;
+            lds[col * PITCH + row] = val;
+        }
+    }
+    __syncthreads();
+    if (K < 2) return;
+
+    f32x4 a_cur[RTILES][4];
+    auto load_a = [&](f32x4 (&dst)[RTILES][4], int r, int kc) {
+        const Tin* base = mats_b + (size_t)r * D * D + (size_t)(row0 + m) * D + kc * 32 + h * 16;
+#pragma unroll
+        for (int i = 0; i < RTILES; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dst[i][q] = load4(base + (size_t)i * 32 * D + q * 4);
+    };
+    load_a(a_cur, K - 2, 0);
+
+    int cur = 0;
+    for (int r = K - 2; r >= 0; --r) {
+        f32x16 acc[RTILES][CTILES];
+#pragma unroll
+        for (int i = 0; i < RTILES; ++i)
+#pragma unroll
+            for (int j = 0; j < CTILES; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+        const float* st = lds + cur * (CB * PITCH);
+#pragma unroll
+        for (int kc = 0; kc < NCH; ++kc) {
+            f32x4 a_nxt[RTILES][4];
+            if (kc + 1 < NCH) {
+                load_a(a_nxt, r, kc + 1);
+            } else if (r > 0) {
+                load_a(a_nxt, r - 1, 0);
+            } else {
+#pragma unroll
+                for (int i = 0; i < RTILES; ++i)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) a_nxt[i][q] = a_cur[i][q];
+            }
+            f32x4 bfrag[CTILES][4];
+#pragma unroll
+            for (int j = 0; j < CTILES; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    bfrag[j][q] = *reinterpret_cast<const f32x4*>(
+                        st + (j * 32 + m) * PITCH + kc * 32 + h * 16 + q * 4);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int i = 0; i < RTILES; ++i)
+#pragma unroll
+                        for (int j = 0; j < CTILES; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                                a_cur[i][q][t], bfrag[j][q][t], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < RTILES; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) a_cur[i][q] = a_nxt[i][q];
+        }
+
+        float* o_r = out_b + (size_t)r * D * D;
+        float* st_new = lds + (cur ^ 1) * (CB * PITCH);
+#pragma unroll
+        for (int i = 0; i < RTILES; ++i)
+#pragma unroll
+            for (int j = 0; j < CTILES; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int row = row0 + i * 32 + g * 8 + h * 4;
+                    const int col = j * 32 + m;
+                    f32x4 v4 = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                                acc[i][j][4 * g + 3]};
+                    *reinterpret_cast<f32x4*>(st_new + col * PITCH + row) = v4;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) o_r[(size_t)(row + t) * D + c0 + col] = v4[t];
+                }
+        __syncthreads();
+        cur ^= 1;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Generic path: any d (small or not a multiple of 32).  Scalar FMA; the column block
+// of the running suffix lives in LDS as S[k][col], double buffered.
+// ---------------------------------------------------------------------------------------
+template <typename Tin>
+__global__ __launch_bounds__(256) void scan_generic_kernel(
+    const Tin* __restrict__ mats, float* __restrict__ out, int B, int K, int d, int cb, int nb) {
+    extern __shared__ __align__(16) float lds[];  // [2][d][cb]
+    const int b = blockIdx.x / nb;
+    const int c0 = (blockIdx.x % nb) * cb;
+    const int ncol = min(cb, d - c0);
+    const int tid = threadIdx.x;
+    const Tin* mats_b = mats + (size_t)b * K * d * d;
+    float* out_b = out + (size_t)b * (K + 1) * d * d;
+    const int nelem = d * ncol;
+
+    {
+        const Tin* a_last = mats_b + (size_t)(K - 1) * d * d;
+        float* o_last = out_b + (size_t)(K - 1) * d * d;
+        float* o_eye = out_b + (size_t)K * d * d;
+        for (int idx = tid; idx < nelem; idx += 256) {
+            const int row = idx / ncol;
+            const int col = idx % ncol;
+            const float val = to_f32(a_last[(size_t)row * d + c0 + col]);
+            o_last[(size_t)row * d + c0 + col] = val;
+            o_eye[(size_t)row * d + c0 + col] = (row == c0 + col) ? 1.0f : 0.0f;
+            lds[row * cb + col] = val;
+        }
+    }
+    __syncthreads();
+
+    int cur = 0;
+    for (int r = K - 2; r >= 0; --r) {
+        const Tin* a = mats_b + (size_t)r * d * d;
+        float* o_r = out_b + (size_t)r * d * d;
+        const float* s_old = lds + cur * d * cb;
+        float* s_new = lds + (cur ^ 1) * d * cb;
+        for (int idx = tid; idx < nelem; idx += 256) {
+            const int row = idx / ncol;
+            const int col = idx % ncol;
+            const Tin* a_row = a + (size_t)row * d;
+            float acc = 0.0f;
+            for (int k = 0; k < d; ++k) acc = fmaf(to_f32(a_row[k]), s_old[k * cb + col], acc);
+            s_new[row * cb + col] = acc;
+            o_r[(size_t)row * d + c0 + col] = acc;
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+}
+
+// K == 0: the result is just the identity.
+__global__ void identity_kernel(float* __restrict__ out, int64_t n_mats, int d) {
+    const int64_t total = n_mats * d * d;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int rc = (int)(idx % ((int64_t)d * d));
+        out[idx] = (rc / d == rc % d) ? 1.0f : 0.0f;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Cotangent chain: one workgroup per batch element, one mat-vec per step.  A wave
+// takes rows wave, wave+NW, ...; lanes run along k so every load instruction reads
+// contiguous memory; the 64 partial sums are folded with a butterfly.  The vector
+// lives in LDS, double buffered, so a step costs one barrier.  HBM-bound: each
+// matrix is read exactly once.
+// ---------------------------------------------------------------------------------------
+template <typename Tin, bool VEC4>
+__global__ __launch_bounds__(512) void cotangent_kernel(
+    const Tin* __restrict__ mats, const float* __restrict__ g, float* __restrict__ out, int K, int d) {
+    extern __shared__ __align__(16) float lds[];  // [2][dpad]
+    const int dpad = (d + 3) & ~3;
+    const int b = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int nw = blockDim.x >> 6;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const Tin* mats_b = mats + (size_t)b * K * d * d;
+    float* out_b = out + (size_t)b * (K + 1) * d;
+
+    for (int i = tid; i < d; i += blockDim.x) {
+        const float val = g[(size_t)b * d + i];
+        lds[i] = val;
+        out_b[(size_t)K * d + i] = val;
+    }
+    __syncthreads();
+
+    int cur = 0;
+    for (int r = K - 1; r >= 0; --r) {
+        const Tin* a = mats_b + (size_t)r * d * d;
+        const float* v_old = lds + cur * dpad;
+        float* v_new = lds + (cur ^ 1) * dpad;
+        for (int row = wave; row < d; row += nw) {
+            const Tin* a_row = a + (size_t)row * d;
+            float acc = 0.0f;
+            if (VEC4) {
+                for (int k = lane * 4; k < d; k += 256) {
+                    const f32x4 a4 = load4(a_row + k);
+                    const f32x4 v4 = *reinterpret_cast<const f32x4*>(v_old + k);
+                    acc = fmaf(a4[0], v4[0], acc);
+                    acc = fmaf(a4[1], v4[1], acc);
+                    acc = fmaf(a4[2], v4[2], acc);
+                    acc = fmaf(a4[3], v4[3], acc);
+                }
+            } else {
+                for (int k = lane; k < d; k += 64) acc = fmaf(to_f32(a_row[k]), v_old[k], acc);
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+            if (lane == 0) {
+                v_new[row] = acc;
+                out_b[(size_t)r * d + row] = acc;
+            }
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+}
+
+template <typename Tin, int D, int RT, int CB>
+int launch_mfma(const void* mats, void* out, int B, int K, hipStream_t stream) {
+    constexpr int NW = D / RT;
+    constexpr int NB = D / CB;
+    constexpr size_t lds_bytes = (size_t)2 * CB * (D + 4) * sizeof(float);
+    auto kern = scan_mfma_kernel<Tin, D, RT, CB>;
+    if (lds_bytes > 64 * 1024) {
+        static thread_local bool attr_done[16] = {};
+        int dev = 0;
+        LBI_HIP_CHECK(hipGetDevice(&dev));
+        if (dev >= 16 || !attr_done[dev]) {
+            LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+            if (dev < 16) attr_done[dev] = true;
+        }
+    }
+    const int groups = (B + 7) / 8;
+    const dim3 grid(groups * 8 * NB);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds_bytes, stream, static_cast<const Tin*>(mats),
+                       static_cast<float*>(out), B, K);
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+template <typename Tin>
+int launch_scan(const void* mats, void* out, int B, int K, int d, hipStream_t stream) {
+    switch (d) {
+        case 256: return launch_mfma<Tin, 256, 64, 64>(mats, out, B, K, stream);
+        case 128: return launch_mfma<Tin, 128, 32, 32>(mats, out, B, K, stream);
+        case 64: return launch_mfma<Tin, 64, 32, 32>(mats, out, B, K, stream);
+        case 32: return launch_mfma<Tin, 32, 32, 32>(mats, out, B, K, stream);
+        default: break;
+    }
+    // Generic: widest column block (<= 32) whose two LDS copies fit in 64 KiB.
+    int cb = d < 32 ? d : 32;
+    while (cb > 1 && (size_t)2 * d * cb * sizeof(float) > 64 * 1024) cb >>= 1;
+    const size_t lds_bytes = (size_t)2 * d * cb * sizeof(float);
+    if (lds_bytes > 64 * 1024) return fail(LBI_ERR_UNSUPPORTED, "suffix scan: d=%d is too large (max 8192)", d);
+    const int nb = (d + cb - 1) / cb;
+    hipLaunchKernelGGL(scan_generic_kernel<Tin>, dim3((unsigned)B * nb), dim3(256), lds_bytes, stream,
+                       static_cast<const Tin*>(mats), static_cast<float*>(out), B, K, d, cb, nb);
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+template <typename Tin>
+int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, int d, hipStream_t stream) {
+    const int dpad = (d + 3) & ~3;
+    const size_t lds_bytes = (size_t)2 * dpad * sizeof(float);
+    if (lds_bytes > 64 * 1024) return fail(LBI_ERR_UNSUPPORTED, "suffix cotangents: d=%d is too large (max 8192)", d);
+    const int threads = d >= 128 ? 512 : (d >= 32 ? 256 : 64);
+    if (d % 4 == 0)
+        hipLaunchKernelGGL((cotangent_kernel<Tin, true>), dim3(B), dim3(threads), lds_bytes, stream,
+                           static_cast<const Tin*>(mats), static_cast<const float*>(g),
+                           static_cast<float*>(out), K, d);
+    else
+        hipLaunchKernelGGL((cotangent_kernel<Tin, false>), dim3(B), dim3(threads), lds_bytes, stream,
+                           static_cast<const Tin*>(mats), static_cast<const float*>(g),
+                           static_cast<float*>(out), K, d);
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+int check_scan_args(const char* what, const void* mats, const void* out, int64_t B, int64_t K, int64_t d,
+                    int in_dtype) {
+    if (B < 0 || K < 0 || d < 0) return fail(LBI_ERR_INVALID, "%s: negative size (B=%lld K=%lld d=%lld)", what,
+                                              (long long)B, (long long)K, (long long)d);
+    if (in_dtype != LBI_F32 && in_dtype != LBI_F16 && in_dtype != LBI_BF16)
+        return fail(LBI_ERR_INVALID, "%s: mats must have float, half, or bfloat16 dtype (got %d)", what, in_dtype);
+    if (B > (1 << 20) || K > (1 << 24) || d > 8192)
+        return fail(LBI_ERR_UNSUPPORTED, "%s: size out of range (B=%lld K=%lld d=%lld)", what, (long long)B,
+                    (long long)K, (long long)d);
+    if ((double)B * (double)(K + 1) * (double)d * (double)d > 9.0e15)
+        return fail(LBI_ERR_UNSUPPORTED, "%s: element count overflows", what);
+    if (B > 0 && d > 0) {
+        if (!out) return fail(LBI_ERR_INVALID, "%s: out is null", what);
+        if (K > 0 && !mats) return fail(LBI_ERR_INVALID, "%s: mats is null", what);
+    }
+    return LBI_OK;
+}
+
+}  // namespace
+}  // namespace lbi
+
+extern "C" int lbi_suffix_scan(const void* mats, void* out, int64_t B, int64_t K, int64_t d, int in_dtype,
+                               int out_dtype, void* stream_v) {
+    using namespace lbi;
+    clear_error();
+    if (int rc = check_scan_args("lbi_suffix_scan", mats, out, B, K, d, in_dtype)) return rc;
+    if (out_dtype != LBI_F32) return fail(LBI_ERR_UNSUPPORTED, "lbi_suffix_scan: out_dtype must be LBI_F32");
+    if (B == 0 || d == 0) return LBI_OK;
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    if (K == 0) {
+        const int64_t total = B * d * d;
+        const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+        hipLaunchKernelGGL(identity_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<float*>(out), B,
+                           (int)d);
+        LBI_HIP_CHECK(hipGetLastError());
+        return LBI_OK;
+    }
+    switch (in_dtype) {
+        case LBI_F32: return launch_scan<float>(mats, out, (int)B, (int)K, (int)d, stream);
+        case LBI_F16: return launch_scan<_Float16>(mats, out, (int)B, (int)K, (int)d, stream);
+        default: return launch_scan<bf16_raw>(mats, out, (int)B, (int)K, (int)d, stream);
+    }
+}
+
+extern "C" int lbi_suffix_cotangents(const void* mats, const void* g, void* out, int64_t B, int64_t K, int64_t d,
+                                     int in_dtype, void* stream_v) {
+    using namespace lbi;
+    clear_error();
+    if (int rc = check_scan_args("lbi_suffix_cotangents", mats, out, B, K, d, in_dtype)) return rc;
+    if (B == 0 || d == 0) return LBI_OK;
+    if (!g) return fail(LBI_ERR_INVALID, "lbi_suffix_cotangents: g is null");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    switch (in_dtype) {
+        case LBI_F32: return launch_cotangent<float>(mats, g, out, (int)B, (int)K, (int)d, stream);
+        case LBI_F16: return launch_cotangent<_Float16>(mats, g, out, (int)B, (int)K, (int)d, stream);
+        default: return launch_cotangent<bf16_raw>(mats, g, out, (int)B, (int)K, (int)d, stream);
+    }
+}

@@ -1,0 +1,73 @@
+"""Suffix scan of interface pullback matrices on the GPU.
+
+Counterpart of reference cuda/interface/__init__.py: same function name, argument
+and result (``[B, K, d, d] -> [B, K+1, d, d]``, fp32 result as the native
+reference extension returns, cuda/interface/suffix_scan.cu:76,110).  The work is
+done by ``lbi_suffix_scan`` / ``lbi_suffix_cotangents`` of liblbi_hip.so.
+"""
+from __future__ import annotations
+
+import torch
+
+from ... import _lib
+
+
+def _validate(mats: torch.Tensor) -> tuple[int, int, int]:
+    # Same contract and messages as reference cuda/interface/__init__.py:12-16 and
+    # cuda/interface/suffix_scan.cu:8-17.
+    if not isinstance(mats, torch.Tensor):
+        raise TypeError("mats must be a torch.Tensor")
+    if mats.dim() != 4:
+        raise ValueError("mats must have shape [B, K, R, R]")
+    bsz, count, rank, rank2 = mats.shape
+    if rank != rank2:
+        raise ValueError("mats must be square in the last two dimensions")
+    if not mats.is_cuda:
+        raise RuntimeError("mats must be a CUDA tensor (this build has no CPU execution path)")
+    if mats.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        raise RuntimeError("mats must have float, half, or bfloat16 dtype")
+    return bsz, count, rank
+
+
+def suffix_scan_pullbacks(mats: torch.Tensor) -> torch.Tensor:
+    """``out[:, r] = mats[:, r] @ ... @ mats[:, K-1]``, ``out[:, K] = I``; fp32, input untouched."""
+    bsz, count, rank = _validate(mats)
+    mats = mats.contiguous()
+    out = torch.empty((bsz, count + 1, rank, rank), device=mats.device, dtype=torch.float32)
+    if out.numel() == 0:
+        return out
+    lib = _lib.load()
+    with torch.cuda.device(mats.device):
+        status = lib.lbi_suffix_scan(
+            mats.data_ptr(), out.data_ptr(), bsz, count, rank,
+            _lib.dtype_code(mats.dtype), _lib.LBI_F32, _lib.current_stream_ptr(mats.device),
+        )
+    _lib.check(status, "lbi_suffix_scan")
+    return out
+
+
+def suffix_scan_cotangents(mats: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """Cotangent-only chain: ``out[:, K] = g``, ``out[:, r] = mats[:, r] @ out[:, r+1]``.
+
+    Returns ``[B, K+1, d]`` fp32 without forming any ``d x d`` product.  Equals
+    ``suffix_scan_pullbacks(mats) @ g`` (reference backward/suffix_scan.py:41-56).
+    """
+    bsz, count, rank = _validate(mats)
+    if g.dim() != 2 or g.shape[0] != bsz or g.shape[1] != rank:
+        raise ValueError("g must have shape [B, R]")
+    mats = mats.contiguous()
+    g32 = g.to(device=mats.device, dtype=torch.float32).contiguous()
+    out = torch.empty((bsz, count + 1, rank), device=mats.device, dtype=torch.float32)
+    if out.numel() == 0:
+        return out
+    lib = _lib.load()
+    with torch.cuda.device(mats.device):
+        status = lib.lbi_suffix_cotangents(
+            mats.data_ptr(), g32.data_ptr(), out.data_ptr(), bsz, count, rank,
+            _lib.dtype_code(mats.dtype), _lib.current_stream_ptr(mats.device),
+        )
+    _lib.check(status, "lbi_suffix_cotangents")
+    return out
+
+
+__all__ = ["suffix_scan_pullbacks", "suffix_scan_cotangents"]

@@ -1,0 +1,63 @@
+"""The C ABI: the built library loads without a GPU and exports what include/lbi_hip.h declares."""
+from __future__ import annotations
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from latent_bounded_interfaces_amd import _lib
+
+HEADER = Path(__file__).resolve().parents[1] / "include" / "lbi_hip.h"
+
+
+def _declared_symbols() -> list[str]:
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(lbi_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_declares_entry_points():
+    names = _declared_symbols()
+    assert {"lbi_suffix_scan", "lbi_suffix_cotangents", "lbi_attn_pullback",
+            "lbi_attn_pullback_workspace_bytes", "lbi_last_error", "lbi_abi_version"} <= set(names)
+
+
+def test_binding_table_matches_header():
+    assert sorted(_lib.SYMBOLS) == _declared_symbols()
+
+
+def test_library_exports_every_declared_symbol():
+    if not _lib.LIB_PATH.exists():
+        pytest.fail(f"{_lib.LIB_PATH} is not built; run python -m latent_bounded_interfaces_amd.build")
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in _declared_symbols():
+        assert hasattr(lib, name), f"{name} missing from liblbi_hip.so"
+    assert _lib.load().lbi_abi_version() == _lib.ABI_VERSION
+
+
+def test_argument_validation_needs_no_gpu():
+    """Contract violations are rejected on the host before any HIP call."""
+    lib = _lib.load()
+    assert lib.lbi_suffix_scan(None, None, -1, 2, 4, _lib.LBI_F32, _lib.LBI_F32, None) == -1
+    assert b"negative" in lib.lbi_last_error()
+    assert lib.lbi_suffix_scan(None, None, 1, 2, 4, 7, _lib.LBI_F32, None) == -1
+    assert b"dtype" in lib.lbi_last_error()
+    assert lib.lbi_suffix_scan(None, None, 1, 2, 4, _lib.LBI_F32, _lib.LBI_F32, None) == -1
+    assert b"null" in lib.lbi_last_error()
+    assert lib.lbi_suffix_scan(None, None, 0, 2, 4, _lib.LBI_F32, _lib.LBI_F32, None) == 0
+    assert lib.lbi_last_error() == b""
+    assert lib.lbi_suffix_cotangents(None, None, None, 1, 2, 4, _lib.LBI_F32, None) == -1
+
+
+def test_wrappers_reject_bad_input_before_touching_the_device():
+    import torch
+
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks
+
+    with pytest.raises(ValueError, match=r"\[B, K, R, R\]"):
+        suffix_scan_pullbacks(torch.zeros(2, 3, 4))
+    with pytest.raises(ValueError, match="square"):
+        suffix_scan_pullbacks(torch.zeros(2, 3, 4, 5))
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        suffix_scan_pullbacks(torch.zeros(2, 3, 4, 4))

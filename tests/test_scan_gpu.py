@@ -1,0 +1,179 @@
+"""Parity of the HIP suffix scan against the CPU oracle, through the C ABI (needs the GPU)."""
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+import pytest
+import torch
+
+from oracle import scan as oscan
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "scan_known_answers.json").read_text())
+
+# Every shape of the reference's tests (tests/test_interface_scan.py:45-53 and :78-86)
+# plus ragged / non-power-of-two cases and each MFMA width with K not a power of two.
+SHAPES = [
+    (1, 0, 1), (1, 1, 1), (1, 1, 4), (2, 3, 5), (2, 4, 8), (4, 8, 16), (1, 16, 64),
+    (1, 2, 16), (2, 4, 32), (2, 8, 64), (1, 16, 128), (1, 8, 256),
+    (4, 8, 32), (3, 5, 32), (9, 7, 64), (5, 3, 128), (3, 5, 256), (2, 6, 48), (2, 3, 33), (1, 4, 100),
+    (17, 2, 256), (1, 1, 256), (2, 0, 32),
+]
+
+
+def _rel_err(actual: torch.Tensor, truth: torch.Tensor) -> float:
+    """max over suffix matrices of max|diff| / max|truth| (fp64 truth)."""
+    diff = (actual.double() - truth).abs().flatten(2).max(dim=2).values
+    ref = truth.abs().flatten(2).max(dim=2).values.clamp_min(1e-30)
+    return float((diff / ref).max())
+
+
+def _scan(mats_cpu: torch.Tensor, device) -> torch.Tensor:
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks
+
+    mats = mats_cpu.to(device)
+    keep = mats.clone()
+    out = suffix_scan_pullbacks(mats)
+    torch.cuda.synchronize()
+    assert torch.equal(mats, keep), "input was modified"
+    return out.cpu()
+
+
+def test_known_answer_2x2(device):
+    case = GOLDEN["order_case_2x2"]
+    out = _scan(torch.tensor(case["mats"], dtype=torch.float32), device)
+    assert torch.equal(out, torch.tensor(case["suffix"], dtype=torch.float32))
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fp32_matches_oracle(shape, device):
+    bsz, count, rank = shape
+    mats, _ = oscan.make_scan_inputs(bsz, count, rank, kind="randn", seed=0)
+    out = _scan(mats, device)
+    assert out.shape == (bsz, count + 1, rank, rank)
+    assert out.dtype == torch.float32
+    assert torch.equal(out[:, count], torch.eye(rank).expand(bsz, rank, rank))
+    truth = oscan.suffix_scan_sequential(mats, dtype=torch.float64)
+    assert _rel_err(out, truth) <= 1e-5  # bar for the fp32 scan
+    # The reference's CPU algorithm (log-depth order) agrees to the same bar.
+    levels = oscan.suffix_scan_levels(mats)
+    assert _rel_err(out, levels.double()) <= 1e-5
+    # Sequential fp32 product has the SAME association order as the kernel.
+    seq = oscan.suffix_scan_sequential(mats)
+    assert torch.allclose(out, seq, atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 8, 64), (2, 5, 256), (3, 4, 24), (2, 6, 128), (2, 9, 32)])
+def test_low_precision_storage_promotes_to_fp32(shape, dtype, device):
+    # reference tests/test_interface_scan.py:104-115
+    bsz, count, rank = shape
+    mats, _ = oscan.make_scan_inputs(bsz, count, rank, kind="randn", seed=0)
+    mats = mats.to(dtype)
+    out = _scan(mats, device)
+    assert out.dtype == torch.float32
+    truth = oscan.suffix_scan_sequential(mats.float(), dtype=torch.float64)
+    # Inputs are rounded before both sides see them, so only fp32 accumulation differs.
+    assert _rel_err(out, truth) <= 1e-5
+    assert torch.allclose(out, oscan.suffix_scan_sequential(mats.float()), atol=2e-1, rtol=5e-3)
+
+
+def test_permutations_are_exact(device):
+    gen = torch.Generator().manual_seed(5)
+    rank, count = 64, 9
+    perms = [torch.randperm(rank, generator=gen) for _ in range(count)]
+    mats = torch.stack([torch.eye(rank)[p] for p in perms]).unsqueeze(0).repeat(3, 1, 1, 1)
+    out = _scan(mats, device)
+    idx = torch.arange(rank)
+    for r in range(count - 1, -1, -1):
+        idx = idx[perms[r]]
+        assert torch.equal(out[1, r], torch.eye(rank)[idx])
+
+
+@pytest.mark.parametrize("shape", [(1, 0, 3), (2, 1, 8), (3, 5, 7), (4, 8, 32), (2, 6, 64), (3, 9, 128),
+                                   (5, 12, 256), (2, 3, 100), (2, 4, 260)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cotangent_chain_matches_oracle(shape, dtype, device):
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents
+
+    bsz, count, rank = shape
+    mats, g = oscan.make_scan_inputs(bsz, count, rank, kind="randn", seed=1)
+    mats = mats.to(dtype)
+    out = suffix_scan_cotangents(mats.to(device), g.to(device)).cpu()
+    assert out.shape == (bsz, count + 1, rank) and out.dtype == torch.float32
+    assert torch.equal(out[:, count], g)
+    truth = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+    scale = truth.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+    assert float(((out.double() - truth).abs() / scale).max()) <= 1e-5
+    case = GOLDEN["order_case_2x2"]
+    got = suffix_scan_cotangents(torch.tensor(case["mats"]).to(device), torch.tensor(case["g"]).to(device))
+    assert torch.equal(got.cpu(), torch.tensor(case["cotangents"]))
+
+
+def test_benchmark_shape_properties(device):
+    """B=64, K=128, d=256: size-independent checks (recurrence, identity tail, reruns bit-stable)."""
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents, suffix_scan_pullbacks
+
+    bsz, count, rank = 64, 128, 256
+    mats, g = oscan.make_scan_inputs(bsz, count, rank, kind="near_identity", seed=0)
+    mats_d = mats.to(device)
+    out = suffix_scan_pullbacks(mats_d)
+    again = suffix_scan_pullbacks(mats_d)
+    assert torch.equal(out, again), "reruns differ"
+    assert torch.equal(out[:, count], torch.eye(rank, device=device).expand(bsz, rank, rank))
+    # out[r] == mats[r] @ out[r+1] for a sample of r, checked in fp64 on the device.
+    for r in (0, 1, 63, 126, 127):
+        want = torch.matmul(mats_d[:, r].double(), out[:, r + 1].double())
+        err = (out[:, r].double() - want).abs().amax() / want.abs().amax()
+        assert float(err) <= 2e-6, (r, float(err))
+    # Full fp64 truth for two batch elements on the CPU.
+    pick = [0, 37]
+    truth = oscan.suffix_scan_sequential(mats[pick], dtype=torch.float64)
+    assert _rel_err(out[pick].cpu(), truth) <= 1e-5
+    # Cotangents: chain == suffix matrices applied to g (the reference's interface_scan_rms check,
+    # backward/scan.py:63-72, bar 1e-5 RMS).
+    g_d = g.to(device)
+    chain = suffix_scan_cotangents(mats_d, g_d)
+    via_mats = torch.einsum("bkij,bj->bki", out.double(), g_d.double())
+    rms = float(torch.sqrt(((chain.double() - via_mats) ** 2).mean()))
+    assert rms < 1e-5
+    # bf16 storage, fp32 accumulate: within 2e-2 of the fp32 path.
+    out_bf16 = suffix_scan_pullbacks(mats_d.to(torch.bfloat16))
+    rel = (out_bf16 - out).abs().flatten(2).amax(dim=2) / out.abs().flatten(2).amax(dim=2)
+    assert float(rel.max()) <= 2e-2
+
+
+def test_backward_module_contract(device):
+    """Counterpart functions of reference backward/suffix_scan.py keep its edge cases."""
+    from latent_bounded_interfaces_amd.backward import suffix_scan as bs
+
+    mats, g = oscan.make_scan_inputs(3, 5, 16, kind="randn", seed=2)
+    jts = [mats[:, r].to(device) for r in range(5)]
+    g_d = g.to(device)
+    suffix = bs.compose_suffix_jacobian_t(jts)
+    assert len(suffix) == 6 and all(s.shape == (3, 16, 16) and s.is_contiguous() for s in suffix)
+    truth = oscan.suffix_scan_sequential(mats, dtype=torch.float64)
+    assert _rel_err(torch.stack([s.cpu() for s in suffix], 1), truth) <= 1e-5
+    assert bs.compose_suffix_jacobian_t([]) == []
+    with pytest.raises(ValueError):
+        bs.compose_suffix_jacobian_t([torch.zeros(2, 3, 4, device=device)])
+    want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+    for flag in (False, True):
+        got = bs.propagate_state_adjoint_with_jacobian_scan(jts, g_d, materialize_suffix=flag)
+        assert len(got) == 6
+        assert torch.allclose(torch.stack([x.cpu() for x in got], 1).double(), want, atol=1e-5, rtol=1e-5)
+    # Drop-last rule and the 0 / 1 region cases.
+    got = bs.propagate_state_adjoint_from_last_region_input(jts, g_d, num_regions=5)
+    want4 = oscan.suffix_cotangents_sequential(mats[:, :4].double(), g.double())
+    assert len(got) == 5
+    assert torch.allclose(torch.stack([x.cpu() for x in got], 1).double(), want4, atol=1e-5, rtol=1e-5)
+    assert bs.propagate_state_adjoint_from_last_region_input([], g_d, num_regions=0) == []
+    assert bs.propagate_state_adjoint_from_last_region_input(jts[:1], g_d, num_regions=1)[0] is g_d
+    with pytest.raises(ValueError):
+        bs.propagate_state_adjoint_from_last_region_input(jts, g_d, num_regions=4)
+    one = bs.apply_jacobian_t(jts[0], g_d)
+    assert torch.allclose(one.cpu(), torch.einsum("bij,bj->bi", mats[:, 0], g), atol=1e-5, rtol=1e-5)
+    stats = bs.interface_state_jacobian_t_stats(jts, include_suffix=True)
+    assert {"jac_local_spec_mean", "jac_suffix_spec_max"} <= set(stats)
