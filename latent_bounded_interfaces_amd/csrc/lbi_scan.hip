@@ -83,18 +83,35 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     __syncthreads();
     if (K < 2) return;
 
-    f32x4 a_cur[RTILES][4];
-    auto load_a = [&](f32x4 (&dst)[RTILES][4], int r, int kc) {
-        const Tin* base = mats_b + (size_t)r * D * D + (size_t)(row0 + m) * D + kc * 32 + h * 16;
+    // Lane's slice of mats[r]: rows row0 + 32*i + m, k = 32*kc + 16*h + [0, 16).
+    auto load_a = [&](f32x4 (&dst)[RTILES][4], const Tin* base) {
 #pragma unroll
         for (int i = 0; i < RTILES; ++i)
 #pragma unroll
             for (int q = 0; q < 4; ++q) dst[i][q] = load4(base + (size_t)i * 32 * D + q * 4);
     };
-    load_a(a_cur, K - 2, 0);
+    const Tin* a_lane = mats_b + (size_t)(row0 + m) * D + h * 16;  // + r*D*D + kc*32
+
+    // mats chunks are prefetched RING-1 chunks ahead into a register ring; the ring
+    // index of a chunk is kc % RING, the same in every step because RING divides NCH.
+    constexpr int RING = (NCH % 4 == 0) ? 4 : 2;
+    constexpr int AHEAD = RING - 1;
+    f32x4 a_ring[RING][RTILES][4];
+    // Chunk number c (0 <= c < AHEAD) counted from the start of step K-2; when NCH == 1
+    // chunk 1 is already in the next step.
+#pragma unroll
+    for (int c = 0; c < AHEAD; ++c) {
+        const int rr = (K - 2) - c / NCH;
+        load_a(a_ring[c % RING], a_lane + (size_t)(rr > 0 ? rr : 0) * D * D + (c % NCH) * 32);
+    }
 
     int cur = 0;
-    for (int r = K - 2; r >= 0; --r) {
+    for (int r = K - 2; r >= 0; r -= (NCH == 1 ? 2 : 1)) {
+        // NCH == 1 runs two steps per trip so ring indices stay compile-time constants.
+#pragma unroll
+        for (int sub = 0; sub < (NCH == 1 ? 2 : 1); ++sub) {
+        const int rs = r - sub;
+        if (rs < 0) break;
         f32x16 acc[RTILES][CTILES];
 #pragma unroll
         for (int i = 0; i < RTILES; ++i)
@@ -103,27 +120,26 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-        const float* st = lds + cur * (CB * PITCH);
+        const float* st = lds + cur * (CB * PITCH) + m * PITCH + h * 16;
+        const Tin* a_r = a_lane + (size_t)rs * D * D;
+        // Chunks past the end of this step belong to mats[rs-1] (a harmless re-read of
+        // mats[0] after the very last step).
+        const Tin* a_wrap = a_lane + (size_t)(rs > 0 ? rs - 1 : 0) * D * D;
 #pragma unroll
         for (int kc = 0; kc < NCH; ++kc) {
-            f32x4 a_nxt[RTILES][4];
-            if (kc + 1 < NCH) {
-                load_a(a_nxt, r, kc + 1);
-            } else if (r > 0) {
-                load_a(a_nxt, r - 1, 0);
-            } else {
-#pragma unroll
-                for (int i = 0; i < RTILES; ++i)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) a_nxt[i][q] = a_cur[i][q];
-            }
+            const int slot = (NCH == 1 ? sub : kc) % RING;
+            const int ahead = kc + AHEAD;
+            load_a(a_ring[(slot + AHEAD) % RING], ahead < NCH ? a_r + ahead * 32 : a_wrap + (ahead - NCH) * 32);
             f32x4 bfrag[CTILES][4];
 #pragma unroll
             for (int j = 0; j < CTILES; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    bfrag[j][q] = *reinterpret_cast<const f32x4*>(
-                        st + (j * 32 + m) * PITCH + kc * 32 + h * 16 + q * 4);
+                    bfrag[j][q] = *reinterpret_cast<const f32x4*>(st + j * 32 * PITCH + kc * 32 + q * 4);
+            // Blocked summation: the 32 products of this k chunk are summed in a fresh
+            // accumulator and added to the running total once, so a total takes D/32
+            // roundings at full magnitude per step instead of D/2.
+            f32x16 part[RTILES][CTILES];
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -131,16 +147,25 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
 #pragma unroll
                     for (int i = 0; i < RTILES; ++i)
 #pragma unroll
-                        for (int j = 0; j < CTILES; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                                a_cur[i][q][t], bfrag[j][q][t], acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < CTILES; ++j) {
+                            if (q == 0 && t == 0) {
+#pragma unroll
+                                for (int e = 0; e < 16; ++e) part[i][j][e] = 0.0f;
+                            }
+                            part[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                                a_ring[slot][i][q][t], bfrag[j][q][t], part[i][j], 0, 0, 0);
+                        }
 #pragma unroll
             for (int i = 0; i < RTILES; ++i)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) a_cur[i][q] = a_nxt[i][q];
+                for (int j = 0; j < CTILES; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[i][j][e] += part[i][j][e];
+            // Keep chunks from being interleaved: it only lengthens register live ranges.
+            __builtin_amdgcn_sched_barrier(0);
         }
 
-        float* o_r = out_b + (size_t)r * D * D;
+        float* o_r = out_b + (size_t)rs * D * D;
         float* st_new = lds + (cur ^ 1) * (CB * PITCH);
 #pragma unroll
         for (int i = 0; i < RTILES; ++i)
@@ -158,6 +183,7 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 }
         __syncthreads();
         cur ^= 1;
+        }
     }
 }
 
@@ -308,7 +334,7 @@ int launch_mfma(const void* mats, void* out, int B, int K, hipStream_t stream) {
 template <typename Tin>
 int launch_scan(const void* mats, void* out, int B, int K, int d, hipStream_t stream) {
     switch (d) {
-        case 256: return launch_mfma<Tin, 256, 64, 64>(mats, out, B, K, stream);
+        case 256: return launch_mfma<Tin, 256, 32, 64>(mats, out, B, K, stream);
         case 128: return launch_mfma<Tin, 128, 32, 32>(mats, out, B, K, stream);
         case 64: return launch_mfma<Tin, 64, 32, 32>(mats, out, B, K, stream);
         case 32: return launch_mfma<Tin, 32, 32, 32>(mats, out, B, K, stream);
