@@ -1,0 +1,71 @@
+"""HIP lowering for Transformer region derivative contracts.
+
+Counterpart of reference backends/transformer_cuda.py (``CudaTransformerLowering``)
+and an implementation of the ``TransformerLowering`` protocol of reference
+backends/transformer.py:64-85.
+"""
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from ..hip.transformer import attention_input_pullback_basis as hip_attention_input_pullback_basis
+
+
+class HipTransformerLowering:
+    """HIP lowering for Transformer region derivative contracts."""
+
+    name = "hip"
+
+    def __init__(self, *, reference_lowering: Any | None = None) -> None:
+        # The reference's class can delegate the two region-level methods to its autograd
+        # lowering (allow_reference_fallback=True).  Here a caller may pass any object that
+        # implements them; without one they raise, as the reference does by default.
+        self.reference_lowering = reference_lowering
+        self.allow_reference_fallback = reference_lowering is not None
+
+    def attention_input_pullback_basis(
+        self,
+        *,
+        q: torch.Tensor,
+        k: torch.Tensor,
+        v: torch.Tensor,
+        output_cotangent_basis: torch.Tensor,
+        softmax_scale: float,
+        causal: bool = True,
+        kernel_mode: str = "hip",
+    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Same keyword-only contract as reference backends/transformer_cuda.py:23-43."""
+        return hip_attention_input_pullback_basis(
+            q,
+            k,
+            v,
+            output_cotangent_basis,
+            softmax_scale=float(softmax_scale),
+            causal=causal,
+            use_cuda=True,
+            kernel_mode=kernel_mode,
+        )
+
+    def input_pullback_basis(self, *, backend: Any, cache: Any, output_cotangent_basis: torch.Tensor) -> torch.Tensor:
+        # reference backends/transformer_cuda.py:45-64
+        if output_cotangent_basis.dim() != 4:
+            raise ValueError("output_cotangent_basis must have shape [B, P, T, D]")
+        if self.reference_lowering is not None:
+            return self.reference_lowering.input_pullback_basis(
+                backend=backend, cache=cache, output_cotangent_basis=output_cotangent_basis
+            )
+        raise NotImplementedError(
+            "HipTransformerLowering.input_pullback_basis: the region-level input pullback for "
+            "output_cotangent_basis [B, P, T, D] is not implemented; pass reference_lowering=... "
+            "to delegate it."
+        )
+
+    def parameter_vjp(self, *, backend: Any, cache: Any, output_cotangent: torch.Tensor) -> dict[str, torch.Tensor]:
+        # reference backends/transformer_cuda.py:66-83
+        if self.reference_lowering is not None:
+            return self.reference_lowering.parameter_vjp(backend=backend, cache=cache, output_cotangent=output_cotangent)
+        raise NotImplementedError(
+            "HipTransformerLowering.parameter_vjp is not implemented; pass reference_lowering=... to delegate it."
+        )

@@ -1,9 +1,65 @@
-// Attention input-pullback for P cotangent basis directions (gfx950).
-#include "lbi_common.h"
+// Attention input-pullback for P cotangent basis directions (gfx950): C ABI entry points
+// and the choice between the MFMA kernels and the generic kernels.
+#include "lbi_attn_generic.h"
+#include "lbi_attn_mfma.h"
 
-extern "C" size_t lbi_attn_pullback_workspace_bytes(int64_t, int64_t, int64_t, int64_t, int64_t, int) { return 0; }
+namespace lbi {
+namespace {
 
-extern "C" int lbi_attn_pullback(const void*, const void*, const void*, const void*, void*, void*, void*, void*,
-                                 size_t, int64_t, int64_t, int64_t, int64_t, int64_t, float, int, int, void*) {
-    return lbi::fail(LBI_ERR_UNSUPPORTED, "lbi_attn_pullback: not built yet");
+int check_attn_dims(int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P, int dtype) {
+    if (B < 0 || H < 0 || T < 0 || Dh < 0 || P < 0)
+        return fail(LBI_ERR_INVALID, "lbi_attn_pullback: negative size (B=%lld H=%lld T=%lld Dh=%lld P=%lld)",
+                    (long long)B, (long long)H, (long long)T, (long long)Dh, (long long)P);
+    if (dtype != LBI_F32 && dtype != LBI_F16 && dtype != LBI_BF16)
+        return fail(LBI_ERR_INVALID, "lbi_attn_pullback: dtype must be float, half or bfloat16 (got %d)", dtype);
+    if (B > (1 << 20) || H > (1 << 16) || T > (1 << 24) || Dh > (1 << 16) || P > (1 << 16) ||
+        (double)B * H * T * Dh * (P > 1 ? P : 1) > 1.0e15 || (double)B * H * (P > 1 ? P : 1) > 2.0e9)
+        return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_pullback: size out of range");
+    return LBI_OK;
+}
+
+}  // namespace
+}  // namespace lbi
+
+extern "C" size_t lbi_attn_pullback_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P,
+                                                    int dtype) {
+    using namespace lbi;
+    if (check_attn_dims(B, H, T, Dh, P, dtype) != LBI_OK) return 0;
+    if (B == 0 || H == 0 || T == 0 || Dh == 0 || P == 0) return 0;
+    const size_t floats = attn_mfma::supports((int)T, (int)Dh, dtype) ? attn_mfma::workspace_floats(B, H, T, Dh, P)
+                                                                     : attn_generic::workspace_floats(B, H, T, P);
+    return (floats * sizeof(float) + 255) & ~(size_t)255;
+}
+
+extern "C" int lbi_attn_pullback(const void* q, const void* k, const void* v, const void* d_out, void* dq, void* dk,
+                                 void* dv, void* workspace, size_t workspace_bytes, int64_t B, int64_t H, int64_t T,
+                                 int64_t Dh, int64_t P, float softmax_scale, int causal, int dtype, void* stream_v) {
+    using namespace lbi;
+    clear_error();
+    if (int rc = check_attn_dims(B, H, T, Dh, P, dtype)) return rc;
+    if (B == 0 || H == 0 || T == 0 || Dh == 0 || P == 0) return LBI_OK;
+    if (!q || !k || !v || !d_out || !dq || !dk || !dv) return fail(LBI_ERR_INVALID, "lbi_attn_pullback: null tensor pointer");
+    const size_t need = lbi_attn_pullback_workspace_bytes(B, H, T, Dh, P, dtype);
+    if (!workspace || workspace_bytes < need)
+        return fail(LBI_ERR_WORKSPACE, "lbi_attn_pullback: workspace of %zu bytes needed, %zu given", need,
+                    workspace_bytes);
+    if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return fail(LBI_ERR_WORKSPACE, "lbi_attn_pullback: workspace must be 16-byte aligned");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    float* ws = static_cast<float*>(workspace);
+    const int b = (int)B, h = (int)H, t = (int)T, dh = (int)Dh, p = (int)P;
+    if (attn_mfma::supports(t, dh, dtype)) {
+        const size_t align = dtype_size(dtype) * 8;  // 16-byte vector loads on every row
+        if (reinterpret_cast<uintptr_t>(q) % align || reinterpret_cast<uintptr_t>(k) % align ||
+            reinterpret_cast<uintptr_t>(v) % align || reinterpret_cast<uintptr_t>(d_out) % align)
+            return fail(LBI_ERR_INVALID, "lbi_attn_pullback: tensors must be 16-byte aligned");
+        return dtype == LBI_F16
+                   ? attn_mfma::launch<_Float16>(q, k, v, d_out, dq, dk, dv, ws, b, h, t, dh, p, softmax_scale, causal, stream)
+                   : attn_mfma::launch<bf16_raw>(q, k, v, d_out, dq, dk, dv, ws, b, h, t, dh, p, softmax_scale, causal, stream);
+    }
+    switch (dtype) {
+        case LBI_F32: return attn_generic::launch<float>(q, k, v, d_out, dq, dk, dv, ws, b, h, t, dh, p, softmax_scale, causal, stream);
+        case LBI_F16: return attn_generic::launch<_Float16>(q, k, v, d_out, dq, dk, dv, ws, b, h, t, dh, p, softmax_scale, causal, stream);
+        default: return attn_generic::launch<bf16_raw>(q, k, v, d_out, dq, dk, dv, ws, b, h, t, dh, p, softmax_scale, causal, stream);
+    }
 }

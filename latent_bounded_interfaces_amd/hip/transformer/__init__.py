@@ -1,0 +1,101 @@
+"""Transformer attention input-pullback for P cotangent basis directions on the GPU.
+
+Counterpart of reference cuda/transformer/__init__.py: same function name, arguments
+and result.  ``q, k, v [B, H, T, Dh]`` and ``output_cotangent_basis [B, P, H, T, Dh]``
+give ``(dq, dk, dv)``, each ``[B, P, H, T, Dh]`` in the input dtype; slice ``p`` is the
+attention backward for cotangent ``output_cotangent_basis[:, p]``.
+
+All work is done by ``lbi_attn_pullback`` of liblbi_hip.so, which recomputes the
+softmax statistics itself (the reference wrapper re-runs a flash forward for them,
+cuda/transformer/__init__.py:248-256).  Every ``kernel_mode`` of the reference is
+accepted, with its limit on P, and all of them run the same HIP kernels; ``"hip"``
+is the unrestricted mode.  There is no torch or CPU execution path here.
+"""
+from __future__ import annotations
+
+import torch
+
+from ... import _lib
+
+# kernel_mode -> largest basis size the reference accepts for it (None: any).
+# reference cuda/transformer/__init__.py:104,165,226-228
+_MODE_BASIS_LIMIT = {
+    "hip": None,
+    "fa2_loop": None,
+    "simple": None,
+    "fa2_p1": 1,
+    "fa2_mma_p1": 1,
+    "fa2_mma_pblock4": 4,
+}
+
+
+def _validate(q, k, v, output_cotangent_basis) -> None:
+    # reference cuda/transformer/__init__.py:21-26
+    if q.dim() != 4 or k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k, and v must have matching shape [B, H, T, Dh]")
+    if output_cotangent_basis.dim() != 5:
+        raise ValueError("output_cotangent_basis must have shape [B, P, H, T, Dh]")
+    if output_cotangent_basis.shape[0] != q.shape[0] or output_cotangent_basis.shape[2:] != q.shape[1:]:
+        raise ValueError("output_cotangent_basis must have shape [B, P, H, T, Dh] matching q/k/v")
+
+
+def attention_input_pullback_basis(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    output_cotangent_basis: torch.Tensor,
+    *,
+    softmax_scale: float,
+    causal: bool = True,
+    use_cuda: bool = True,
+    kernel_mode: str = "fa2_mma_pblock4",
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """dQ, dK, dV for every basis direction (signature of reference cuda/transformer/__init__.py:279-289)."""
+    _validate(q, k, v, output_cotangent_basis)
+    if kernel_mode not in _MODE_BASIS_LIMIT:
+        raise ValueError(f"unknown attention pullback kernel_mode: {kernel_mode}")
+    basis = output_cotangent_basis.shape[1]
+    limit = _MODE_BASIS_LIMIT[kernel_mode]
+    if limit == 1 and basis != 1:
+        raise ValueError(f"kernel_mode='{kernel_mode}' requires output_cotangent_basis.shape[1] == 1")
+    if limit == 4 and not 1 <= basis <= 4:
+        raise ValueError("kernel_mode='fa2_mma_pblock4' requires 1 <= output_cotangent_basis.shape[1] <= 4")
+    if not use_cuda:
+        raise RuntimeError(
+            "use_cuda=False selects the reference's dense torch formula, which this build does not ship; "
+            "only the HIP kernels are available"
+        )
+    if not q.is_cuda:
+        raise RuntimeError("q, k, v must be CUDA tensors (this build has no CPU execution path)")
+    if not (k.device == q.device and v.device == q.device and output_cotangent_basis.device == q.device):
+        raise RuntimeError("q, k, v and output_cotangent_basis must be on the same device")
+    if not (k.dtype == q.dtype and v.dtype == q.dtype and output_cotangent_basis.dtype == q.dtype):
+        raise RuntimeError("q, k, v and output_cotangent_basis must have the same dtype")
+    dtype = _lib.dtype_code(q.dtype)
+
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    d_out = output_cotangent_basis.contiguous()
+    bsz, heads, seqlen, head_dim = q.shape
+    dq = torch.empty_like(d_out)
+    dk = torch.empty_like(d_out)
+    dv = torch.empty_like(d_out)
+    if d_out.numel() == 0:
+        return dq, dk, dv
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        need = int(lib.lbi_attn_pullback_workspace_bytes(bsz, heads, seqlen, head_dim, basis, dtype))
+        workspace = torch.empty(max(need, 256), device=q.device, dtype=torch.uint8)
+        status = lib.lbi_attn_pullback(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+            workspace.data_ptr(), workspace.numel(),
+            bsz, heads, seqlen, head_dim, basis,
+            float(softmax_scale), int(bool(causal)), dtype, _lib.current_stream_ptr(q.device),
+        )
+    _lib.check(status, "lbi_attn_pullback")
+    # The workspace is only used by kernels already queued on this stream; torch's
+    # caching allocator reuses it in stream order, so releasing it here is safe.
+    return dq, dk, dv
+
+
+__all__ = ["attention_input_pullback_basis"]

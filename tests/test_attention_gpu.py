@@ -1,0 +1,153 @@
+"""Parity of the HIP attention input-pullback against the CPU oracle, through the C ABI (needs the GPU)."""
+from __future__ import annotations
+
+import json
+import math
+from pathlib import Path
+
+import pytest
+import torch
+
+from oracle import attention as oattn
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "attention_known_answers.json").read_text())
+
+
+def _run(q, k, v, g, device, *, scale, causal, mode="hip"):
+    from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis
+
+    args = [t.to(device) for t in (q, k, v, g)]
+    keep = [t.clone() for t in args]
+    out = attention_input_pullback_basis(*args, softmax_scale=scale, causal=causal, kernel_mode=mode)
+    torch.cuda.synchronize()
+    for a, b in zip(args, keep):
+        assert torch.equal(a, b), "input was modified"
+    return tuple(t.cpu() for t in out)
+
+
+def _max_rel(actual, truth):
+    """max|diff| / max|truth| over a whole tensor."""
+    return float((actual.double() - truth.double()).abs().max() / truth.double().abs().max().clamp_min(1e-30))
+
+
+@pytest.mark.parametrize("case", ["two_keys_equal", "single_token"])
+def test_known_answers(case, device):
+    c = GOLDEN[case]
+    q, k, v, g = (torch.tensor(c[n], dtype=torch.float32) for n in ("q", "k", "v", "d_out"))
+    got = _run(q, k, v, g, device, scale=c["softmax_scale"], causal=c["causal"])
+    for name, t in zip(("dq", "dk", "dv"), got):
+        assert torch.allclose(t, torch.tensor(c[name]), atol=1e-6), name
+
+
+# fp32 cases of the reference's tests (tests/test_cuda_attention_pullback.py:62-66, 86-90, 115-119)
+# plus ragged ones (T not a multiple of the 16-wide tile, odd head dims, T=1).
+FP32_CASES = [
+    (101, (2, 3, 5, 4), 2), (103, (1, 2, 4, 3), 3), (117, (1, 2, 4, 16), 3),
+    (5, (1, 1, 1, 8), 2), (6, (2, 2, 17, 5), 1), (7, (1, 3, 33, 24), 2), (8, (1, 2, 40, 72), 3),
+    (9, (1, 1, 64, 64), 2), (10, (1, 2, 19, 130), 1),
+]
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("seed,shape,basis", FP32_CASES)
+def test_fp32_matches_oracle(seed, shape, basis, causal, device):
+    torch.manual_seed(seed)
+    q = torch.randn(*shape)
+    k = torch.randn_like(q)
+    v = torch.randn_like(q)
+    g = torch.randn(shape[0], basis, *shape[1:])
+    scale = 1.0 / math.sqrt(shape[-1])
+    got = _run(q, k, v, g, device, scale=scale, causal=causal)
+    want = oattn.attention_pullback_sdpa_loop(q, k, v, g, softmax_scale=scale, causal=causal)
+    truth = oattn.attention_pullback_dense(q, k, v, g, softmax_scale=scale, causal=causal, dtype=torch.float64)
+    for a, b, c in zip(got, want, truth):
+        assert a.shape == g.shape and a.dtype == torch.float32
+        assert torch.allclose(a, b, atol=2e-5, rtol=2e-5)  # the reference's fp32 bar
+        assert torch.allclose(a.double(), c, atol=2e-5, rtol=2e-5)
+
+
+# 16-bit storage: the MFMA kernels (T % 64 == 0, Dh in {64, 128}) and the generic ones otherwise.
+# (121, (1, 2, 16, 64), P) are the reference's fp16 cases (tests/test_cuda_attention_pullback.py:178-243);
+# (8, 8, 128, 64) with P=4 is the reference benchmark shape.
+LOWP_CASES = [
+    (121, (1, 2, 16, 64), 1), (129, (1, 2, 16, 64), 4), (11, (2, 2, 64, 64), 2), (12, (1, 3, 128, 128), 3),
+    (13, (2, 1, 192, 64), 5), (14, (1, 2, 320, 128), 2), (15, (1, 1, 576, 128), 1), (16, (8, 8, 128, 64), 4),
+    (17, (1, 2, 96, 64), 2), (18, (1, 1, 64, 32), 2),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("seed,shape,basis", LOWP_CASES)
+def test_low_precision_matches_oracle(seed, shape, basis, causal, dtype, device):
+    q, k, v, g = oattn.make_attention_inputs(*shape, basis, dtype=dtype, seed=seed)
+    scale = 1.0 / math.sqrt(shape[-1])
+    got = _run(q, k, v, g, device, scale=scale, causal=causal)
+    # fp32 path on the same (already rounded) inputs
+    truth = oattn.attention_pullback_blocked(q, k, v, g, softmax_scale=scale, causal=causal, dtype=torch.float32)
+    for name, a, c in zip(("dq", "dk", "dv"), got, truth):
+        assert a.shape == g.shape and a.dtype == dtype
+        assert _max_rel(a, c) <= 2e-2, (name, _max_rel(a, c))  # bar: <= 2e-2 against the fp32 path
+        assert torch.allclose(a.float(), c, atol=3e-2 * float(c.abs().max()), rtol=3e-2), name
+
+
+def test_modes_and_contract(device):
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+    from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis
+
+    q, k, v, g = (t.to(device) for t in oattn.make_attention_inputs(1, 2, 16, 64, 4, dtype=torch.float16, seed=131))
+    scale = 0.125
+    base = attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, kernel_mode="hip")
+    for mode in ("fa2_loop", "simple", "fa2_mma_pblock4"):
+        out = attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, kernel_mode=mode)
+        assert all(torch.equal(a, b) for a, b in zip(out, base))
+    # P limits of the reference's modes (tests/test_cuda_attention_pullback.py:163-173, 281-291)
+    for mode in ("fa2_p1", "fa2_mma_p1"):
+        with pytest.raises(ValueError, match="== 1"):
+            attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, kernel_mode=mode)
+        one = attention_input_pullback_basis(q, k, v, g[:, :1], softmax_scale=scale, kernel_mode=mode)
+        assert all(torch.equal(a, b[:, :1]) for a, b in zip(one, base))
+    g5 = torch.cat([g, g[:, :1]], dim=1)
+    with pytest.raises(ValueError, match="<= 4"):
+        attention_input_pullback_basis(q, k, v, g5, softmax_scale=scale)
+    with pytest.raises(ValueError, match="unknown attention pullback kernel_mode"):
+        attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, kernel_mode="nope")
+    with pytest.raises(ValueError):
+        attention_input_pullback_basis(q, k[:, :1], v, g, softmax_scale=scale)
+    with pytest.raises(ValueError):
+        attention_input_pullback_basis(q, k, v, g[:, 0], softmax_scale=scale)
+    # lowering wrapper (reference tests/test_cuda_attention_pullback.py:294-315)
+    low = HipTransformerLowering()
+    assert low.name == "hip"
+    out = low.attention_input_pullback_basis(q=q, k=k, v=v, output_cotangent_basis=g5, softmax_scale=scale)
+    assert all(torch.equal(a[:, :4], b) for a, b in zip(out, base))
+    with pytest.raises(NotImplementedError):
+        low.input_pullback_basis(backend=None, cache=None, output_cotangent_basis=torch.zeros(1, 1, 2, 3))
+    with pytest.raises(ValueError):
+        low.input_pullback_basis(backend=None, cache=None, output_cotangent_basis=torch.zeros(1, 2, 3))
+    with pytest.raises(NotImplementedError):
+        low.parameter_vjp(backend=None, cache=None, output_cotangent=torch.zeros(1, 2, 3))
+
+
+def test_long_context_properties(device):
+    """bf16, T=4096, Dh=128, P=16 on two (b, h) slices: size-independent checks."""
+    from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis
+
+    q, k, v, g = (t.to(device) for t in oattn.make_attention_inputs(1, 2, 4096, 128, 16, dtype=torch.bfloat16, seed=0))
+    scale = 1.0 / math.sqrt(128)
+    dq, dk, dv = attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, kernel_mode="hip")
+    again = attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, kernel_mode="hip")
+    assert all(torch.equal(a, b) for a, b in zip((dq, dk, dv), again)), "reruns differ"
+    # basis independence: direction p alone gives the same slice
+    solo = attention_input_pullback_basis(q, k, v, g[:, 5:6].contiguous(), softmax_scale=scale, kernel_mode="hip")
+    for a, b in zip(solo, (dq, dk, dv)):
+        assert _max_rel(a[:, 0], b[:, 5].float()) <= 2e-2
+    # first query row attends one key: dQ there is zero; P=1 slice equals torch's own attention backward
+    assert float(dq[:, :, :, 0].abs().max()) == 0.0
+    qr, kr, vr = (t.float().requires_grad_(True) for t in (q, k, v))
+    out = torch.nn.functional.scaled_dot_product_attention(qr, kr, vr, is_causal=True, scale=scale)
+    want = torch.autograd.grad(out, (qr, kr, vr), grad_outputs=g[:, 3].float())
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), want):
+        assert _max_rel(a[:, 3], b) <= 2e-2, (name, _max_rel(a[:, 3], b))
