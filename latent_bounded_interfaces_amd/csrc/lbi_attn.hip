@@ -2,6 +2,7 @@
 // and the choice between the MFMA kernels and the generic kernels.
 #include "lbi_attn_generic.h"
 #include "lbi_attn_mfma.h"
+#include "lbi_attn_dkdv128.h"
 
 namespace lbi {
 namespace {

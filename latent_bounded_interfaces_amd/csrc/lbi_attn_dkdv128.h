@@ -1,0 +1,310 @@
+// dK/dV kernel of the attention input-pullback for head dim 128 (fp16 / bf16 storage).
+//
+// Same ownership and arithmetic as attn_mfma::dkdv_kernel (one wave = 64 keys x one
+// direction, workgroup = 256 keys, Q and d_out_p streamed in 32-query tiles), with the
+// data path rebuilt around what the counters showed: the first version spent as many
+// cycles in VALU work and in waits as in MFMA.
+//
+//  * Q / d_out tiles and the lse2 / delta rows go global -> LDS with global_load_lds
+//    (16 bytes per lane, no staging registers, no ds_write), one tile ahead, into a
+//    two-stage ring.  The loop is unrolled by two so the stage is a compile-time
+//    immediate of every LDS read.
+//  * The XOR swizzle is linear over GF(2), so every LDS address is
+//    (lane constant) ^ (compile-time constant) + immediate: one VALU op per read at most.
+//  * Causal masking runs only in the first 8 steps of a workgroup (queries that
+//    are not past all of its 256 keys); the main loop has no compare / select.
+//  * The products are ordered S, dP, [P], dV, [dS], dK so the VALU phase in brackets
+//    has independent MFMA work on either side to overlap with.
+#pragma once
+
+#include <type_traits>
+
+#include "lbi_attn_mfma.h"
+
+namespace lbi {
+namespace attn_mfma {
+
+// s_waitcnt immediate with only vmcnt constrained (gfx9 encoding: vmcnt = [15:14|3:0],
+// expcnt [6:4], lgkmcnt [11:8]).
+constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+// 64 lanes x 16 bytes, global -> LDS.  Lane l reads 16 bytes at base + voff(l) and the
+// data lands at lds_base + 16*l.  lds_base must be wave-uniform and below 64 KiB.
+__device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voff), "s"(base)
+                 : "memory");
+}
+
+template <typename T, bool CAUSAL>
+__global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                      const T* __restrict__ v, const T* __restrict__ d_out,
+                                                      const float* __restrict__ lse2, const float* __restrict__ delta,
+                                                      T* __restrict__ dk, T* __restrict__ dv, int n_bh, int H, int P,
+                                                      int T_len, float scale) {
+    constexpr int DH = 128, KS = 8, ND = 4;
+    constexpr unsigned TILE = 32 * DH * 2;         // 8 KiB
+    constexpr unsigned STATS = 4 * 256;            // per wave: 32 lse2 + 32 delta floats
+    constexpr unsigned STAGE = 2 * TILE + STATS;   // Q tile, d_out tile, stats
+    constexpr int NDMA = 5;                        // global_load_lds per wave per tile
+    extern __shared__ __align__(16) char smem[];   // [2][STAGE]
+
+    const int n_kb = (T_len + 255) / 256;
+    int bh, rem;
+    if (!map_block(n_kb * P, n_bh, bh, rem)) return;
+    const int p = rem / n_kb;
+    const int kb = rem % n_kb;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 31, h = lane >> 5;
+    const bool active = kb * 256 + wave * 64 < T_len;
+    const int j0w = min(kb * 256 + wave * 64, T_len - 64);
+    const size_t base = (size_t)bh * T_len * DH;
+    const size_t prow = (((size_t)b * P + p) * H + hh) * T_len;
+    const T* q_bh = q + base;
+    const T* g_p = d_out + prow * DH;
+    const float* lse_bh = lse2 + (size_t)bh * T_len;
+    const float* delta_p = delta + prow;
+
+    // ---- lane constants of the LDS addressing -------------------------------------------
+    const unsigned lane_nat = m * 256 + ((h ^ swz<DH>(m)) << 4);  // ^ (ks << 5)
+    const unsigned s16 = lane & 15, g1 = (lane >> 4) & 1;
+    const unsigned lane_phys = (((s16 >> 2) & 3) << 2) | ((2 * g1 + ((s16 & 3) >> 1)) ^ h);
+    const unsigned lane_tr = (4 * h + (s16 >> 2)) * 256 + (lane_phys << 4) + ((s16 & 1) << 3);  // ^ (nd<<6 | hi<<5)
+    const unsigned lane_stat = (unsigned)wave * 256 + 16 * h;  // + 32*g (lse2), + 128 (delta)
+
+    // ---- global -> LDS: this wave's share of a tile step ---------------------------------
+    // Tile slot sigma = 64u + lane (u = 2*wave, 2*wave+1): row sigma/16, physical chunk sigma%16.
+    unsigned dma_off[2];
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        const int r = 4 * (2 * wave + x) + (lane >> 4);
+        dma_off[x] = r * 256 + (((lane & 15) ^ swz<DH>(r)) << 4);
+    }
+    // lanes 0-7: lse2 float4 #lane, lanes 8-15: delta float4 #(lane-8), as offsets from lse_bh
+    const unsigned stat_off =
+        (lane < 8 ? 0u : (unsigned)((const char*)delta_p - (const char*)lse_bh)) + 16 * (lane & 7);
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
+    auto issue_tile = [&](int i_row, unsigned stage_base) __attribute__((always_inline)) {
+        const unsigned row_bytes = (unsigned)i_row * 256;
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            dma16(q_bh, row_bytes + dma_off[x], lds0 + stage_base + 1024 * (2 * wave + x));
+            dma16(g_p, row_bytes + dma_off[x], lds0 + stage_base + TILE + 1024 * (2 * wave + x));
+        }
+        // Every wave keeps its own copy of the 64 row statistics: no cross-wave dependency.
+        if (lane < 16) dma16(lse_bh, (unsigned)i_row * 4 + stat_off, lds0 + stage_base + 2 * TILE + 256 * wave);
+    };
+
+    // K of this wave's 64 keys stays in registers (B operand of S).  V of the same keys sits
+    // in LDS behind the two stages, as two swizzled 32-row tiles per wave: registers hold
+    // the 256 accumulators, K, and the S / dP tiles of a step, and no more.
+    u32x4 kf[2][KS];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            kf[t][ks] = *reinterpret_cast<const u32x4*>(k + base + (size_t)(j0w + 32 * t + m) * DH + 16 * ks + 8 * h);
+    {
+        char* vt_w = smem + 2 * STAGE + wave * 2 * TILE;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int slot = 64 * u + lane;  // 16-byte slot of the wave's 64 x 256-byte block
+            const int r = slot >> 4, c = slot & 15;
+            const u32x4 val = *reinterpret_cast<const u32x4*>(v + base + (size_t)(j0w + r) * DH + 8 * c);
+            *reinterpret_cast<u32x4*>(vt_w + (r >> 5) * TILE + tile_off<DH>(r & 31, c)) = val;
+        }
+    }
+    const char* vt = smem + 2 * STAGE + wave * 2 * TILE;
+    f32x16 acc_k[2][ND], acc_v[2][ND];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int nd = 0; nd < ND; ++nd) {
+            acc_k[t][nd] = zero16();
+            acc_v[t][nd] = zero16();
+        }
+    const float sc2 = scale * LOG2E;
+
+    // One tile step on the stage at byte offset SB.  thr: element (t, 8g+e) is above the
+    // diagonal iff 8g + e < thr + 32t.
+    // LDS operand reads are written a block ahead of their use so their latency can pass
+    // under the products of the block before.
+    auto lds16 = [&](const char* p) __attribute__((always_inline)) {
+        return *reinterpret_cast<const u32x4*>(p);
+    };
+    auto lds_f4 = [&](const char* p) __attribute__((always_inline)) {
+        return *reinterpret_cast<const f32x4*>(p);
+    };
+    auto tr_frag = [&](const char* tile, int kk, int nd) __attribute__((always_inline)) {
+        typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+        const s16x4 lo =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + (lane_tr ^ (nd << 6)) + (16 * kk) * 256));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_ptr)(tile + (lane_tr ^ ((nd << 6) | 32)) + (16 * kk + 8) * 256));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        return u32x4{l2[0], l2[1], h2[0], h2[1]};
+    };
+
+    // One tile step on the stage at byte offset SB.  thr: element (t, 8g+e) is above the
+    // diagonal iff 8g + e < thr + 32t.
+    auto step = [&](auto mask_tag, auto stage_tag, int thr) __attribute__((always_inline)) {
+        constexpr bool MASK = decltype(mask_tag)::value;
+        constexpr unsigned SB = decltype(stage_tag)::value;
+        const char* qt = smem + SB;
+        const char* gt = smem + SB + TILE;
+        const char* st = smem + SB + 2 * TILE;
+
+        // ---- S = Q K^T: all eight Q fragments in flight at once, then the first dP operands.
+        u32x4 qa[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qa[ks] = lds16(qt + (lane_nat ^ (ks << 5)));
+        u32x4 ga[2], va[2], vb[2];  // dP operands of block ks live in slot ks & 1
+        ga[0] = lds16(gt + lane_nat);
+        va[0] = lds16(vt + lane_nat);
+        vb[0] = lds16(vt + TILE + lane_nat);
+        f32x16 s[2];
+        s[0] = Mma<T>::mma_v_start(qa[0], kf[0][0]);
+        s[1] = Mma<T>::mma_v_start(qa[0], kf[1][0]);
+#pragma unroll
+        for (int ks = 1; ks < KS; ++ks) {
+            Mma<T>::mma_v(qa[ks], kf[0][ks], s[0]);
+            Mma<T>::mma_v(qa[ks], kf[1][ks], s[1]);
+        }
+        f32x4 l4 = lds_f4(st + lane_stat);
+        mma_v_settle(s[0], s[1]);
+
+        // ---- dP = dO V^T, with the P phase (exp2, mask, pack) of one (g, t) block of S after
+        // each pair of products: independent work, so it runs while the matrix pipe is busy.
+        f32x16 dp[2];
+        u32x4 pa[2][2], dsa[2][2];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if (ks + 1 < KS) {
+                ga[nxt] = lds16(gt + (lane_nat ^ ((ks + 1) << 5)));
+                va[nxt] = lds16(vt + (lane_nat ^ ((ks + 1) << 5)));
+                vb[nxt] = lds16(vt + TILE + (lane_nat ^ ((ks + 1) << 5)));
+            }
+            if (ks == 0) {
+                dp[0] = Mma<T>::mma_v_start(ga[cur], va[cur]);
+                dp[1] = Mma<T>::mma_v_start(ga[cur], vb[cur]);
+            } else {
+                Mma<T>::mma_v(ga[cur], va[cur], dp[0]);
+                Mma<T>::mma_v(ga[cur], vb[cur], dp[1]);
+            }
+            const int g = ks >> 1, t = ks & 1;
+            float pr[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                pr[e] = __builtin_amdgcn_exp2f(s[t][4 * g + e] * sc2 - l4[e]);
+                if (MASK && (8 * g + e < thr + 32 * t)) pr[e] = 0.0f;
+            }
+            unsigned w0 = Mma<T>::pack2(pr[0], pr[1]), w1 = Mma<T>::pack2(pr[2], pr[3]);
+            if (t == 1 && g < 3) l4 = lds_f4(st + lane_stat + 32 * (g + 1));
+            pin_here(w0, w1);
+            pa[t][g >> 1][2 * (g & 1)] = w0;
+            pa[t][g >> 1][2 * (g & 1) + 1] = w1;
+        }
+        f32x4 d4 = lds_f4(st + lane_stat + 128);
+        u32x4 bfr[2];  // tr fragments of step i live in slot i & 1
+        bfr[0] = tr_frag(gt, 0, 0);
+        mma_v_settle(dp[0], dp[1]);
+
+        // ---- dV += P^T dO (needs P only), with the dS phase of one (g, t) block after each pair.
+#pragma unroll
+        for (int i = 0; i < 2 * ND; ++i) {
+            const int kk = i / ND, nd = i % ND, cur = i & 1;
+            bfr[cur ^ 1] = (i + 1 < 2 * ND) ? tr_frag(gt, (i + 1) / ND, (i + 1) % ND) : tr_frag(qt, 0, 0);
+            acc_v[0][nd] = Mma<T>::mma(pa[0][kk], bfr[cur], acc_v[0][nd]);
+            acc_v[1][nd] = Mma<T>::mma(pa[1][kk], bfr[cur], acc_v[1][nd]);
+            const int g = i >> 1, t = i & 1;
+            const unsigned p0 = pa[t][g >> 1][2 * (g & 1)], p1 = pa[t][g >> 1][2 * (g & 1) + 1];
+            const float d0 = Mma<T>::lo(p0) * (dp[t][4 * g + 0] - d4[0]);
+            const float d1 = Mma<T>::hi(p0) * (dp[t][4 * g + 1] - d4[1]);
+            const float d2 = Mma<T>::lo(p1) * (dp[t][4 * g + 2] - d4[2]);
+            const float d3 = Mma<T>::hi(p1) * (dp[t][4 * g + 3] - d4[3]);
+            unsigned w0 = Mma<T>::pack2(d0, d1), w1 = Mma<T>::pack2(d2, d3);
+            if (t == 1 && g < 3) d4 = lds_f4(st + lane_stat + 128 + 32 * (g + 1));
+            pin_here(w0, w1);
+            dsa[t][g >> 1][2 * (g & 1)] = w0;
+            dsa[t][g >> 1][2 * (g & 1) + 1] = w1;
+        }
+
+        // ---- dK += dS^T Q
+#pragma unroll
+        for (int i = 0; i < 2 * ND; ++i) {
+            const int kk = i / ND, nd = i % ND, cur = i & 1;
+            if (i + 1 < 2 * ND) bfr[cur ^ 1] = tr_frag(qt, (i + 1) / ND, (i + 1) % ND);
+            acc_k[0][nd] = Mma<T>::mma(dsa[0][kk], bfr[cur], acc_k[0][nd]);
+            acc_k[1][nd] = Mma<T>::mma(dsa[1][kk], bfr[cur], acc_k[1][nd]);
+        }
+    };
+
+    const int i_begin = CAUSAL ? kb * 256 : 0;
+    const int n_it = (T_len - i_begin) / 32;             // even: T_len % 64 == 0
+    const int n_mask = CAUSAL ? min(8, n_it) : 0;         // steps that can touch the diagonal
+    issue_tile(i_begin, 0);
+    // One trip = two tile steps (stage 0 then stage 1).  Before a step: this wave's share of
+    // the tile has landed (all but the newest NDMA loads done), then the barrier makes
+    // everyone's share visible and retires the other stage, which is refilled at once.
+    auto two_steps = [&](auto mask_tag, int it) __attribute__((always_inline)) {
+        const int i0 = i_begin + it * 32;
+        const int thr = j0w + m - 4 * h - i0;
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        __syncthreads();
+        issue_tile(min(i0 + 32, T_len - 32), STAGE);
+        step(mask_tag, std::integral_constant<unsigned, 0>{}, thr);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        __syncthreads();
+        issue_tile(min(i0 + 64, T_len - 32), 0);
+        step(mask_tag, std::integral_constant<unsigned, STAGE>{}, thr - 32);
+    };
+    int it = 0;
+    for (; it < n_mask; it += 2) two_steps(std::true_type{}, it);
+    for (; it < n_it; it += 2) two_steps(std::false_type{}, it);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    (void)NDMA;
+
+    if (active) {
+        unsigned short* ok = reinterpret_cast<unsigned short*>(dk + (prow + j0w) * DH);
+        unsigned short* ov = reinterpret_cast<unsigned short*>(dv + (prow + j0w) * DH);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int nd = 0; nd < ND; ++nd)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    const unsigned k2 = Mma<T>::pack2(acc_k[t][nd][r] * scale, acc_k[t][nd][r + 1] * scale);
+                    const unsigned v2 = Mma<T>::pack2(acc_v[t][nd][r], acc_v[t][nd][r + 1]);
+                    const size_t o0 = (size_t)(32 * t + c_row(r, h)) * DH + 32 * nd + m;
+                    const size_t o1 = (size_t)(32 * t + c_row(r + 1, h)) * DH + 32 * nd + m;
+                    ok[o0] = (unsigned short)(k2 & 0xffffu);
+                    ok[o1] = (unsigned short)(k2 >> 16);
+                    ov[o0] = (unsigned short)(v2 & 0xffffu);
+                    ov[o1] = (unsigned short)(v2 >> 16);
+                }
+    }
+}
+
+constexpr size_t dkdv128_lds_bytes = 2 * (2 * 32 * 128 * 2 + 4 * 256) + 4 * 2 * 32 * 128 * 2;  // stages + V
+
+template <typename T, int DH, bool CAUSAL>
+void launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
+                 int n_bh, int H, int P, int T_len, float scale, hipStream_t stream) {
+    const int n_kb = (T_len + 255) / 256;
+    if constexpr (DH == 128) {
+        static_assert(dkdv128_lds_bytes <= 160 * 1024, "LDS budget");
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dkdv128_kernel<T, CAUSAL>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkdv128_lds_bytes);
+        hipLaunchKernelGGL((dkdv128_kernel<T, CAUSAL>), dim3(grid_size(n_kb * P, n_bh)), dim3(256), dkdv128_lds_bytes,
+                           stream, q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale);
+    } else {
+        constexpr size_t lds_bytes = 4 * 32 * DH * 2 + 2 * 64 * sizeof(float);
+        hipLaunchKernelGGL((dkdv_kernel<T, DH, CAUSAL>), dim3(grid_size(n_kb * P, n_bh)), dim3(256), lds_bytes, stream,
+                           q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale);
+    }
+}
+
+}  // namespace attn_mfma
+}  // namespace lbi

@@ -37,8 +37,31 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr float LOG2E = 1.4426950408889634f;
 
+// Scheduling fence between the phases of a tile step: keeps the compiler from
+// interleaving phases, which only lengthens live ranges in these register-bound loops.
+#ifndef LBI_ATTN_FENCE
+#define LBI_ATTN_FENCE 1
+#endif
+#if LBI_ATTN_FENCE
+#define LBI_PHASE_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define LBI_PHASE_FENCE() ((void)0)
+#endif
+
 template <typename T> struct Mma;
 template <> struct Mma<bf16_raw> {
+    // Same product with the 32 x 32 result tile in ordinary VGPRs ("vgprcd" form).  The
+    // compiler puts every builtin MFMA result in the 256 accumulation registers; a kernel
+    // whose long-lived accumulators already fill those needs its short-lived S / dP tiles
+    // elsewhere, or it shuffles registers on every step.  start(): C = 0.
+    static __device__ __forceinline__ f32x16 mma_v_start(u32x4 a, u32x4 b) {
+        f32x16 d;
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+        return d;
+    }
+    static __device__ __forceinline__ void mma_v(u32x4 a, u32x4 b, f32x16& c) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
     static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w << 16); }
     static __device__ __forceinline__ float hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
     static __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
@@ -52,6 +75,14 @@ template <> struct Mma<bf16_raw> {
     }
 };
 template <> struct Mma<_Float16> {
+    static __device__ __forceinline__ f32x16 mma_v_start(u32x4 a, u32x4 b) {
+        f32x16 d;
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+        return d;
+    }
+    static __device__ __forceinline__ void mma_v(u32x4 a, u32x4 b, f32x16& c) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
     static __device__ __forceinline__ float lo(unsigned w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
     static __device__ __forceinline__ float hi(unsigned w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
     static __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
@@ -126,6 +157,19 @@ template <typename T> __device__ __forceinline__ u32x4 pack_frag(const f32x16& c
     return u32x4{Mma<T>::pack2(c[8 * kk + 0], c[8 * kk + 1]), Mma<T>::pack2(c[8 * kk + 2], c[8 * kk + 3]),
                  Mma<T>::pack2(c[8 * kk + 4], c[8 * kk + 5]), Mma<T>::pack2(c[8 * kk + 6], c[8 * kk + 7])};
 }
+
+// The matrix pipe hands a VGPR-form result to the vector ALU only some cycles after issue,
+// and nothing stalls an early reader.  The compiler pads its own MFMAs; after the ones
+// issued through Mma<T>::mma_v the padding is explicit: 16 idle issue slots cover the
+// 8-pass products used here.
+__device__ __forceinline__ void mma_v_settle(f32x16& c0, f32x16& c1) {
+    asm volatile("s_nop 15" : "+v"(c0), "+v"(c1));
+}
+
+// Pins the instructions that produce w0, w1 before this point in program order (the asm
+// MFMAs are volatile too, so VALU work written between two of them stays between them
+// and runs while the matrix pipe is busy).
+__device__ __forceinline__ void pin_here(unsigned& w0, unsigned& w1) { asm volatile("" : "+v"(w0), "+v"(w1)); }
 
 __device__ __forceinline__ f32x16 zero16() {
     f32x16 z;
@@ -375,7 +419,7 @@ __global__ __launch_bounds__(256) void dq_kernel(const T* __restrict__ q, const 
                 pq[g >> 1][2 * (g & 1)] = Mma<T>::pack2(pr[0], pr[1]);
                 pq[g >> 1][2 * (g & 1) + 1] = Mma<T>::pack2(pr[2], pr[3]);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            LBI_PHASE_FENCE();
             f32x16 dp[PB];
 #pragma unroll
             for (int pp = 0; pp < PB; ++pp) dp[pp] = zero16();
@@ -398,7 +442,7 @@ __global__ __launch_bounds__(256) void dq_kernel(const T* __restrict__ q, const 
                     dsa[pp][g >> 1][2 * (g & 1)] = Mma<T>::pack2(d0, d1);
                     dsa[pp][g >> 1][2 * (g & 1) + 1] = Mma<T>::pack2(d2, d3);
                 }
-            __builtin_amdgcn_sched_barrier(0);
+            LBI_PHASE_FENCE();
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
@@ -487,20 +531,30 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const T* __restrict__ q, cons
 
     const int i_begin = CAUSAL ? kb * 256 : 0;
     const int n_it = (T_len - i_begin) / 32;
+    // The 32 lse2 and 32 delta values of a query tile travel with it through LDS
+    // (threads 0-7 carry lse2, 8-15 delta, one float4 each).
+    float* row_stats = reinterpret_cast<float*>(smem + 4 * TILE_BYTES);  // [2][64]
+    const float* stat_src = (tid < 8 ? lse_bh : delta_p) + 4 * (tid & 7);
+    f32x4 stat_reg = {0.0f, 0.0f, 0.0f, 0.0f};
     TileLoader<DH> ql, gl;
     ql.fetch(q_bh, i_begin, tid);
     gl.fetch(g_p, i_begin, tid);
+    if (tid < 16) stat_reg = *reinterpret_cast<const f32x4*>(stat_src + i_begin);
     ql.commit(smem, tid);
     gl.commit(smem + TILE_BYTES, tid);
+    if (tid < 16) *reinterpret_cast<f32x4*>(row_stats + 4 * tid) = stat_reg;
     __syncthreads();
     for (int it = 0; it < n_it; ++it) {
         const int i0 = i_begin + it * 32;
         const char* qt = smem + (it & 1) * 2 * TILE_BYTES;
         const char* gt = qt + TILE_BYTES;
+        const float* lse_t = row_stats + (it & 1) * 64;
+        const float* delta_t = lse_t + 32;
         {
             const int i_next = min(i0 + 32, T_len - 32);
             ql.fetch(q_bh, i_next, tid);
             gl.fetch(g_p, i_next, tid);
+            if (tid < 16) stat_reg = *reinterpret_cast<const f32x4*>(stat_src + i_next);
         }
         {
             // Query tiles wholly before this wave's keys get P = 0 and add nothing.
@@ -517,7 +571,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const T* __restrict__ q, cons
             u32x4 pa[2][2], dsa[2][2];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_bh + i0 + 8 * g + 4 * h);
+                const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_t + 8 * g + 4 * h);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
                     float pr[4];
@@ -530,7 +584,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const T* __restrict__ q, cons
                     pa[t][g >> 1][2 * (g & 1) + 1] = Mma<T>::pack2(pr[2], pr[3]);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
+            LBI_PHASE_FENCE();
             f32x16 dp[2] = {zero16(), zero16()};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -540,7 +594,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const T* __restrict__ q, cons
             }
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_p + i0 + 8 * g + 4 * h);
+                const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_t + 8 * g + 4 * h);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
                     const unsigned w0 = pa[t][g >> 1][2 * (g & 1)], w1 = pa[t][g >> 1][2 * (g & 1) + 1];
@@ -552,7 +606,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const T* __restrict__ q, cons
                     dsa[t][g >> 1][2 * (g & 1) + 1] = Mma<T>::pack2(d2, d3);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
+            LBI_PHASE_FENCE();
             // tr fragments are fetched one (kk, nd) step ahead of the products that use them.
             u32x4 bg = frag_tr<DH>(gt, lane, 0, 0), bq = frag_tr<DH>(qt, lane, 0, 0);
 #pragma unroll
@@ -570,13 +624,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const T* __restrict__ q, cons
                 }
                 bg = bg_n;
                 bq = bq_n;
-                __builtin_amdgcn_sched_barrier(0);
+                LBI_PHASE_FENCE();
             }
         }
         {
             char* nxt = smem + ((it + 1) & 1) * 2 * TILE_BYTES;
             ql.commit(nxt, tid);
             gl.commit(nxt + TILE_BYTES, tid);
+            if (tid < 16) *reinterpret_cast<f32x4*>(row_stats + ((it + 1) & 1) * 64 + 4 * tid) = stat_reg;
         }
         __syncthreads();
     }
@@ -610,11 +665,17 @@ inline size_t workspace_floats(int64_t B, int64_t H, int64_t T, int64_t Dh, int6
     return (size_t)(B * H * T + B * P * H * T + B * H * T * Dh);
 }
 
+// dK/dV launch: head dim 128 has its own kernel (lbi_attn_dkdv128.h).
+template <typename T, int DH, bool CAUSAL>
+void launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
+                 int n_bh, int H, int P, int T_len, float scale, hipStream_t stream);
+
 template <typename T, int DH, bool CAUSAL>
 int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T* dv, float* workspace, int B,
                  int H, int T_len, int P, float scale, hipStream_t stream) {
     constexpr int PB = DH == 128 ? 2 : 4;
     constexpr size_t lds_bytes = 4 * 32 * DH * 2;
+    constexpr size_t lds_bytes_dkdv = lds_bytes + 2 * 64 * sizeof(float);
     const int n_bh = B * H;
     float* lse2 = workspace;
     float* delta = lse2 + (size_t)n_bh * T_len;
@@ -630,8 +691,7 @@ int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T
                        dim3(256), 0, stream, g, o32, delta, H, P, T_len, n_rows);
     hipLaunchKernelGGL((dq_kernel<T, DH, PB, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), lds_bytes,
                        stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
-    hipLaunchKernelGGL((dkdv_kernel<T, DH, CAUSAL>), dim3(grid_size(n_kb * P, n_bh)), dim3(256), lds_bytes, stream, q,
-                       k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale);
+    launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
