@@ -3,8 +3,8 @@
 
 One "step" is one pass of the interface suffix scan at the scale configuration
 (B=64 batch elements, K=128 regions, d=256 interface width, fp32): all K suffix
-matrices (``lbi_suffix_scan``) plus all K suffix cotangents
-(``lbi_suffix_cotangents``), inputs resident in HBM.  ``value`` is composed
+matrices plus all K suffix cotangents, computed by one call of
+``lbi_suffix_scan_with_cotangents``, inputs resident in HBM.  ``value`` is composed
 pullbacks per second, ``B*K / t_step``.
 
 Prints ONE JSON line.  Besides the contract keys it carries
@@ -31,6 +31,12 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 
 SCAN_B, SCAN_K, SCAN_D = 64, 128, 256
 
+# HBM bytes per launch of the scan kernel at this shape, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 1 GiB device
+# copy (FETCH_SIZE reads 0.5 KiB per KiB moved on this part, WRITE_SIZE 1.0):
+# 1 050 100 KiB * 2.0 + 2 113 536 KiB * 1.0.  See profiles/scan_fp32_B64_K128_d256_pmc.md.
+MEASURED_SCAN_TRAFFIC_BYTES = int((1050100 * 2.0 + 2113536 * 1.0) * 1024)
+
 
 def _parse() -> argparse.Namespace:
     ap = argparse.ArgumentParser()
@@ -39,7 +45,10 @@ def _parse() -> argparse.Namespace:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline scan (used for profiling)")
-    ap.add_argument("--cpu-sample-batch", type=int, default=8)
+    ap.add_argument("--cpu-sample-batch", type=int, default=64)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy (a known-size reference for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     return ap.parse_args()
 
 
@@ -125,13 +134,22 @@ def main() -> int:
                                              SCAN_D, _lib.dtype_code(mats.dtype), stream),
                    "lbi_suffix_cotangents")
 
+    if args.copy_calibration:
+        src = torch.empty(256 * 1024 * 1024, device=device, dtype=torch.float32)  # 1 GiB
+        src.fill_(1.0)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
     mats, g = _scan_inputs(device, torch.float32)
     out = torch.empty((SCAN_B, SCAN_K + 1, SCAN_D, SCAN_D), device=device, dtype=torch.float32)
     cot = torch.empty((SCAN_B, SCAN_K + 1, SCAN_D), device=device, dtype=torch.float32)
 
     def step():
-        scan_call(mats, out)
-        cot_call(mats, g, cot)
+        _lib.check(lib.lbi_suffix_scan_with_cotangents(mats.data_ptr(), g.data_ptr(), out.data_ptr(), cot.data_ptr(),
+                                                       SCAN_B, SCAN_K, SCAN_D, _lib.dtype_code(mats.dtype),
+                                                       _lib.LBI_F32, stream), "lbi_suffix_scan_with_cotangents")
 
     # ---- headline: exactly `steps` timed steps between synchronisations ----------------
     for _ in range(args.warmup):
@@ -146,16 +164,16 @@ def main() -> int:
     value = SCAN_B * SCAN_K / (wall / args.steps)
 
     # ---- dominant kernel alone, HIP events on its stream ------------------------------
-    scan_ms = _time_events(lambda: scan_call(mats, out), args.steps, 2)
+    scan_ms = _time_events(step, args.steps, 2)
     scan_avg = statistics.fmean(scan_ms)
     scan_flops = SCAN_B * (SCAN_K - 1) * 2 * SCAN_D ** 3
     scan_bytes = SCAN_B * SCAN_K * SCAN_D * SCAN_D * (4 + 4)
     achieved_tflops = scan_flops / (scan_avg * 1e-3) / 1e12
-    first = out.clone()
-    scan_call(mats, out)
+    first, first_cot = out.clone(), cot.clone()
+    step()
     torch.cuda.synchronize()
-    bit_stable = bool(torch.equal(first, out))
-    del first
+    bit_stable = bool(torch.equal(first, out)) and bool(torch.equal(first_cot, cot))
+    del first, first_cot
 
     result = {
         "metric": "scan composed-pullbacks/s + attn-pullback TFLOP/s, % of MI355X roofline",
@@ -176,12 +194,12 @@ def main() -> int:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "scan_mfma_kernel<float,256,...> (lbi_suffix_scan)",
+            "kernel": "scan_mfma_kernel<float,256,32,64,true> (lbi_suffix_scan_with_cotangents)",
             "achieved": achieved_tflops,
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved_tflops / PEAK_FP32_MFMA_TFLOPS,
-            "traffic": None,
+            "traffic": MEASURED_SCAN_TRAFFIC_BYTES,
             "kernel_ms_avg": scan_avg,
             "kernel_ms_min": min(scan_ms),
             "algorithmic_flops": scan_flops,
@@ -193,6 +211,11 @@ def main() -> int:
 
     if not args.no_extra:
         extra = {}
+        only_ms = _time_events(lambda: scan_call(mats, out), args.steps, 2)
+        extra["scan_matrices_only_fp32"] = {
+            "kernel_ms_avg": statistics.fmean(only_ms),
+            "tflops": scan_flops / (statistics.fmean(only_ms) * 1e-3) / 1e12,
+        }
         cot_ms = _time_events(lambda: cot_call(mats, g, cot), args.steps, 2)
         cot_avg = statistics.fmean(cot_ms)
         cot_bytes = SCAN_B * SCAN_K * SCAN_D * SCAN_D * 4

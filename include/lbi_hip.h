@@ -59,6 +59,20 @@ int lbi_suffix_scan(const void* mats, void* out,
                     int in_dtype, int out_dtype, void* stream);
 
 /*
+ * Suffix scan and cotangent chain in one pass over mats:
+ *
+ *   out as lbi_suffix_scan;  cot [B, K+1, d] (fp32) as lbi_suffix_cotangents for g [B, d] (fp32).
+ *
+ * This is the whole of propagate_state_adjoint_with_jacobian_scan of the reference
+ * (backward/suffix_scan.py:41-56: scan, then K mat-vecs suffix[r] @ g), with the mat-vecs
+ * computed as the chain cot[r] = mats[r] @ cot[r+1] from the operand registers of the
+ * matrix products, i.e. at no extra memory traffic.
+ */
+int lbi_suffix_scan_with_cotangents(const void* mats, const void* g, void* out, void* cot,
+                                    int64_t B, int64_t K, int64_t d,
+                                    int in_dtype, int out_dtype, void* stream);
+
+/*
  * Cotangent-only suffix chain: no d x d product is formed.
  *
  *   mats [B, K, d, d] (in_dtype), g [B, d] (fp32)  ->  out [B, K+1, d] (fp32)

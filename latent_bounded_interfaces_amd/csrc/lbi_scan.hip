@@ -35,9 +35,15 @@ namespace {
 // prefetched one 32-wide k chunk ahead, across step boundaries too (mats do not
 // depend on the running product).  St is double buffered: one barrier per step.
 // ---------------------------------------------------------------------------------------
-template <typename Tin, int D, int RT, int CB>
+//
+// COT: the kernel also runs the cotangent chain v[r] = mats[r] @ v[r+1], v[K] = g.  The
+// fragments of mats[r] that feed the MFMAs are already in registers, so a step costs
+// D/2 extra FMAs per lane (and nothing from HBM); every column block computes the chain,
+// block 0 writes it.
+template <typename Tin, int D, int RT, int CB, bool COT>
 __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
-    const Tin* __restrict__ mats, float* __restrict__ out, int B, int K) {
+    const Tin* __restrict__ mats, float* __restrict__ out, const float* __restrict__ g,
+    float* __restrict__ cot, int B, int K) {
     constexpr int NW = D / RT;          // waves per workgroup
     constexpr int NT = 64 * NW;         // threads
     constexpr int RTILES = RT / 32;
@@ -46,7 +52,8 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     constexpr int PITCH = D + 4;
     constexpr int NCH = D / 32;         // k chunks per step
 
-    extern __shared__ __align__(16) float lds[];  // [2][CB][PITCH]
+    extern __shared__ __align__(16) float lds[];  // [2][CB][PITCH], then (COT) [2][D]
+    float* vbuf = lds + 2 * CB * PITCH;
 
     // Workgroups are dealt round-robin to the 8 XCDs; all column blocks of one
     // batch element get ids that are equal mod 8 so they share one L2.
@@ -78,6 +85,26 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
             o_last[row * D + c0 + col] = val;
             o_eye[row * D + c0 + col] = (row == c0 + col) ? 1.0f : 0.0f;
             lds[col * PITCH + row] = val;
+        }
+        if (COT) {
+            // v[K] = g and v[K-1] = mats[K-1] @ g (one row per thread, once per kernel)
+            const float* g_b = g + (size_t)b * D;
+            float* cot_b = cot + (size_t)b * (K + 1) * D;
+            for (int row = tid; row < D; row += NT) {
+                float acc = 0.0f;
+                for (int k4 = 0; k4 < D; k4 += 4) {
+                    const f32x4 a4 = load4(a_last + row * D + k4);
+                    acc = fmaf(a4[0], g_b[k4], acc);
+                    acc = fmaf(a4[1], g_b[k4 + 1], acc);
+                    acc = fmaf(a4[2], g_b[k4 + 2], acc);
+                    acc = fmaf(a4[3], g_b[k4 + 3], acc);
+                }
+                vbuf[row] = acc;
+                if (c0 == 0) {
+                    cot_b[(size_t)K * D + row] = g_b[row];
+                    cot_b[(size_t)(K - 1) * D + row] = acc;
+                }
+            }
         }
     }
     __syncthreads();
@@ -121,6 +148,10 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
         const float* st = lds + cur * (CB * PITCH) + m * PITCH + h * 16;
+        const float* v_old = vbuf + cur * D + h * 16;
+        float vdot[RTILES];
+#pragma unroll
+        for (int i = 0; i < RTILES; ++i) vdot[i] = 0.0f;
         const Tin* a_r = a_lane + (size_t)rs * D * D;
         // Chunks past the end of this step belong to mats[rs-1] (a harmless re-read of
         // mats[0] after the very last step).
@@ -161,6 +192,16 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 for (int j = 0; j < CTILES; ++j)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) acc[i][j][e] += part[i][j][e];
+            if (COT) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 v4 = *reinterpret_cast<const f32x4*>(v_old + kc * 32 + q * 4);
+#pragma unroll
+                    for (int i = 0; i < RTILES; ++i)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) vdot[i] = fmaf(a_ring[slot][i][q][t], v4[t], vdot[i]);
+                }
+            }
             // Keep chunks from being interleaved: it only lengthens register live ranges.
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -181,6 +222,18 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
 #pragma unroll
                     for (int t = 0; t < 4; ++t) o_r[(size_t)(row + t) * D + c0 + col] = v4[t];
                 }
+        if (COT) {
+            float* v_new = vbuf + (cur ^ 1) * D;
+            float* cot_r = cot + ((size_t)b * (K + 1) + rs) * D;
+#pragma unroll
+            for (int i = 0; i < RTILES; ++i) {
+                const float total = vdot[i] + __shfl_xor(vdot[i], 32, 64);  // the two k halves of a row
+                if (h == 0) {
+                    v_new[row0 + i * 32 + m] = total;
+                    if (c0 == 0) cot_r[row0 + i * 32 + m] = total;
+                }
+            }
+        }
         __syncthreads();
         cur ^= 1;
         }
@@ -307,12 +360,12 @@ __global__ __launch_bounds__(512) void cotangent_kernel(
     }
 }
 
-template <typename Tin, int D, int RT, int CB>
-int launch_mfma(const void* mats, void* out, int B, int K, hipStream_t stream) {
+template <typename Tin, int D, int RT, int CB, bool COT>
+int launch_mfma_cot(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
     constexpr int NW = D / RT;
     constexpr int NB = D / CB;
-    constexpr size_t lds_bytes = (size_t)2 * CB * (D + 4) * sizeof(float);
-    auto kern = scan_mfma_kernel<Tin, D, RT, CB>;
+    constexpr size_t lds_bytes = ((size_t)2 * CB * (D + 4) + (COT ? 2 * D : 0)) * sizeof(float);
+    auto kern = scan_mfma_kernel<Tin, D, RT, CB, COT>;
     if (lds_bytes > 64 * 1024) {
         static thread_local bool attr_done[16] = {};
         int dev = 0;
@@ -326,19 +379,33 @@ int launch_mfma(const void* mats, void* out, int B, int K, hipStream_t stream) {
     const int groups = (B + 7) / 8;
     const dim3 grid(groups * 8 * NB);
     hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds_bytes, stream, static_cast<const Tin*>(mats),
-                       static_cast<float*>(out), B, K);
+                       static_cast<float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), B, K);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
 
+template <typename Tin, int D, int RT, int CB>
+int launch_mfma(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
+    return cot ? launch_mfma_cot<Tin, D, RT, CB, true>(mats, out, g, cot, B, K, stream)
+               : launch_mfma_cot<Tin, D, RT, CB, false>(mats, out, nullptr, nullptr, B, K, stream);
+}
+
 template <typename Tin>
-int launch_scan(const void* mats, void* out, int B, int K, int d, hipStream_t stream) {
+int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, int d, hipStream_t stream);
+
+// g / cot may be null (matrices only).  With them, the MFMA widths run the fused kernel;
+// other widths run the generic scan followed by the cotangent chain kernel.
+template <typename Tin>
+int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, int K, int d, hipStream_t stream) {
     switch (d) {
-        case 256: return launch_mfma<Tin, 256, 32, 64>(mats, out, B, K, stream);
-        case 128: return launch_mfma<Tin, 128, 32, 32>(mats, out, B, K, stream);
-        case 64: return launch_mfma<Tin, 64, 32, 32>(mats, out, B, K, stream);
-        case 32: return launch_mfma<Tin, 32, 32, 32>(mats, out, B, K, stream);
+        case 256: return launch_mfma<Tin, 256, 32, 64>(mats, out, g, cot, B, K, stream);
+        case 128: return launch_mfma<Tin, 128, 32, 32>(mats, out, g, cot, B, K, stream);
+        case 64: return launch_mfma<Tin, 64, 32, 32>(mats, out, g, cot, B, K, stream);
+        case 32: return launch_mfma<Tin, 32, 32, 32>(mats, out, g, cot, B, K, stream);
         default: break;
+    }
+    if (cot) {
+        if (int rc = launch_cotangent<Tin>(mats, g, cot, B, K, d, stream)) return rc;
     }
     // Generic: widest column block (<= 32) whose two LDS copies fit in 64 KiB.
     int cb = d < 32 ? d : 32;
@@ -391,12 +458,14 @@ int check_scan_args(const char* what, const void* mats, const void* out, int64_t
 }  // namespace
 }  // namespace lbi
 
-extern "C" int lbi_suffix_scan(const void* mats, void* out, int64_t B, int64_t K, int64_t d, int in_dtype,
-                               int out_dtype, void* stream_v) {
-    using namespace lbi;
+namespace lbi {
+namespace {
+
+int scan_entry(const char* what, const void* mats, void* out, const void* g, void* cot, int64_t B, int64_t K,
+               int64_t d, int in_dtype, int out_dtype, void* stream_v) {
     clear_error();
-    if (int rc = check_scan_args("lbi_suffix_scan", mats, out, B, K, d, in_dtype)) return rc;
-    if (out_dtype != LBI_F32) return fail(LBI_ERR_UNSUPPORTED, "lbi_suffix_scan: out_dtype must be LBI_F32");
+    if (int rc = check_scan_args(what, mats, out, B, K, d, in_dtype)) return rc;
+    if (out_dtype != LBI_F32) return fail(LBI_ERR_UNSUPPORTED, "%s: out_dtype must be LBI_F32", what);
     if (B == 0 || d == 0) return LBI_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     if (K == 0) {
@@ -405,13 +474,33 @@ extern "C" int lbi_suffix_scan(const void* mats, void* out, int64_t B, int64_t K
         hipLaunchKernelGGL(identity_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<float*>(out), B,
                            (int)d);
         LBI_HIP_CHECK(hipGetLastError());
+        // the chain of zero matrices is just g
+        if (cot) return launch_cotangent<float>(mats, g, cot, (int)B, 0, (int)d, stream);
         return LBI_OK;
     }
     switch (in_dtype) {
-        case LBI_F32: return launch_scan<float>(mats, out, (int)B, (int)K, (int)d, stream);
-        case LBI_F16: return launch_scan<_Float16>(mats, out, (int)B, (int)K, (int)d, stream);
-        default: return launch_scan<bf16_raw>(mats, out, (int)B, (int)K, (int)d, stream);
+        case LBI_F32: return launch_scan<float>(mats, out, g, cot, (int)B, (int)K, (int)d, stream);
+        case LBI_F16: return launch_scan<_Float16>(mats, out, g, cot, (int)B, (int)K, (int)d, stream);
+        default: return launch_scan<bf16_raw>(mats, out, g, cot, (int)B, (int)K, (int)d, stream);
     }
+}
+
+}  // namespace
+}  // namespace lbi
+
+extern "C" int lbi_suffix_scan(const void* mats, void* out, int64_t B, int64_t K, int64_t d, int in_dtype,
+                               int out_dtype, void* stream_v) {
+    return lbi::scan_entry("lbi_suffix_scan", mats, out, nullptr, nullptr, B, K, d, in_dtype, out_dtype, stream_v);
+}
+
+extern "C" int lbi_suffix_scan_with_cotangents(const void* mats, const void* g, void* out, void* cot, int64_t B,
+                                               int64_t K, int64_t d, int in_dtype, int out_dtype, void* stream_v) {
+    using namespace lbi;
+    if (B > 0 && d > 0 && (!g || !cot)) {
+        clear_error();
+        return fail(LBI_ERR_INVALID, "lbi_suffix_scan_with_cotangents: g or cot is null");
+    }
+    return scan_entry("lbi_suffix_scan_with_cotangents", mats, out, g, cot, B, K, d, in_dtype, out_dtype, stream_v);
 }
 
 extern "C" int lbi_suffix_cotangents(const void* mats, const void* g, void* out, int64_t B, int64_t K, int64_t d,

@@ -70,4 +70,26 @@ def suffix_scan_cotangents(mats: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     return out
 
 
-__all__ = ["suffix_scan_pullbacks", "suffix_scan_cotangents"]
+def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Both results of the two functions above from one pass over ``mats`` (one kernel
+    for d in {32, 64, 128, 256}): ``(suffix [B, K+1, d, d], cotangents [B, K+1, d])``, fp32."""
+    bsz, count, rank = _validate(mats)
+    if g.dim() != 2 or g.shape[0] != bsz or g.shape[1] != rank:
+        raise ValueError("g must have shape [B, R]")
+    mats = mats.contiguous()
+    g32 = g.to(device=mats.device, dtype=torch.float32).contiguous()
+    out = torch.empty((bsz, count + 1, rank, rank), device=mats.device, dtype=torch.float32)
+    cot = torch.empty((bsz, count + 1, rank), device=mats.device, dtype=torch.float32)
+    if out.numel() == 0:
+        return out, cot
+    lib = _lib.load()
+    with torch.cuda.device(mats.device):
+        status = lib.lbi_suffix_scan_with_cotangents(
+            mats.data_ptr(), g32.data_ptr(), out.data_ptr(), cot.data_ptr(), bsz, count, rank,
+            _lib.dtype_code(mats.dtype), _lib.LBI_F32, _lib.current_stream_ptr(mats.device),
+        )
+    _lib.check(status, "lbi_suffix_scan_with_cotangents")
+    return out, cot
+
+
+__all__ = ["suffix_scan_pullbacks", "suffix_scan_cotangents", "suffix_scan_pullbacks_and_cotangents"]

@@ -112,6 +112,30 @@ def test_cotangent_chain_matches_oracle(shape, dtype, device):
     assert torch.equal(got.cpu(), torch.tensor(case["cotangents"]))
 
 
+@pytest.mark.parametrize("shape", [(1, 0, 3), (2, 1, 8), (3, 5, 7), (4, 8, 32), (2, 6, 64), (3, 9, 128), (5, 12, 256),
+                                   (9, 1, 256), (2, 2, 32), (2, 3, 100), (1, 1, 64)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_fused_scan_and_cotangents(shape, dtype, device):
+    """One pass giving both results equals the two separate entry points (bit-exact for the
+    matrices) and the oracle for the cotangents."""
+    from latent_bounded_interfaces_amd.hip.interface import (
+        suffix_scan_pullbacks,
+        suffix_scan_pullbacks_and_cotangents,
+    )
+
+    bsz, count, rank = shape
+    mats, g = oscan.make_scan_inputs(bsz, count, rank, kind="randn", seed=4)
+    mats = mats.to(dtype)
+    mats_d, g_d = mats.to(device), g.to(device)
+    out, cot = suffix_scan_pullbacks_and_cotangents(mats_d, g_d)
+    assert torch.equal(out, suffix_scan_pullbacks(mats_d))
+    assert cot.shape == (bsz, count + 1, rank) and cot.dtype == torch.float32
+    assert torch.equal(cot[:, count].cpu(), g)
+    truth = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+    scale = truth.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+    assert float(((cot.cpu().double() - truth).abs() / scale).max()) <= 1e-5
+
+
 def test_benchmark_shape_properties(device):
     """B=64, K=128, d=256: size-independent checks (recurrence, identity tail, reruns bit-stable)."""
     from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents, suffix_scan_pullbacks
@@ -134,11 +158,16 @@ def test_benchmark_shape_properties(device):
     assert _rel_err(out[pick].cpu(), truth) <= 1e-5
     # Cotangents: chain == suffix matrices applied to g (the reference's interface_scan_rms check,
     # backward/scan.py:63-72, bar 1e-5 RMS).
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks_and_cotangents
+
     g_d = g.to(device)
     chain = suffix_scan_cotangents(mats_d, g_d)
     via_mats = torch.einsum("bkij,bj->bki", out.double(), g_d.double())
     rms = float(torch.sqrt(((chain.double() - via_mats) ** 2).mean()))
     assert rms < 1e-5
+    fused_out, fused_cot = suffix_scan_pullbacks_and_cotangents(mats_d, g_d)
+    assert torch.equal(fused_out, out)
+    assert float(torch.sqrt(((fused_cot.double() - via_mats) ** 2).mean())) < 1e-5
     # bf16 storage, fp32 accumulate: inputs are rounded to bf16 before either path sees
     # them; bar 2e-2 against the fp32 path on the same (rounded) inputs.
     mats_bf16 = mats_d.to(torch.bfloat16)
