@@ -34,8 +34,8 @@ SCAN_B, SCAN_K, SCAN_D = 64, 128, 256
 # HBM bytes per launch of the scan kernel at this shape, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 1 GiB device
 # copy (FETCH_SIZE reads 0.5 KiB per KiB moved on this part, WRITE_SIZE 1.0):
-# 1 050 100 KiB * 2.0 + 2 113 536 KiB * 1.0.  See profiles/scan_fp32_B64_K128_d256_pmc.md.
-MEASURED_SCAN_TRAFFIC_BYTES = int((1050100 * 2.0 + 2113536 * 1.0) * 1024)
+# 1 052 300 KiB * 2.0 + 2 121 792 KiB * 1.0.  See profiles/scan_fp32_B64_K128_d256_pmc.md.
+MEASURED_SCAN_TRAFFIC_BYTES = int((1052300 * 2.0 + 2121792 * 1.0) * 1024)
 
 
 def _parse() -> argparse.Namespace:
