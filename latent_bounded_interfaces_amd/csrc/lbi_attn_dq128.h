@@ -1,0 +1,264 @@
+// dQ kernel of the attention input-pullback for head dim 128 (fp16 / bf16 storage).
+//
+// One wave owns 32 queries and PB = 4 directions (the 256 accumulation registers are
+// exactly its four dQ tiles of 32 x 128); a workgroup is 4 waves = 128 queries.
+//   S^T  = K Q^T        A = K tile (LDS, shared), B = Q (registers)   lanes = queries, registers = keys
+//   P    = exp2(S^T c - lse2), once for the four directions
+//   dP^T = V dO_p^T     A = V tile (LDS, shared), B = dO_p (LDS, private to the wave)
+//   dS_p = P (dP_p - delta_p)
+//   dQ_p += dS_p K      A = dS_p (registers), B = K tile through transpose reads
+// K/V tiles of 32 keys arrive by global_load_lds into a two-stage ring (loop unrolled by
+// two, stage offsets are immediates); the wave's four d_out tiles are copied to LDS once.
+// S^T and dP^T tiles use VGPR-form MFMAs; the dS work of direction p is written between
+// the dP products of direction p+1 so it runs while the matrix pipe is busy.  Causal
+// masking is confined to the last four steps of a workgroup.
+#pragma once
+
+#include "lbi_attn_dkdv128.h"
+
+namespace lbi {
+namespace attn_mfma {
+
+template <typename T, bool CAUSAL>
+__global__ __launch_bounds__(256) void dq128_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                    const T* __restrict__ v, const T* __restrict__ d_out,
+                                                    const float* __restrict__ lse2, const float* __restrict__ delta,
+                                                    T* __restrict__ dq, int n_bh, int H, int P, int T_len,
+                                                    float scale) {
+    constexpr int DH = 128, KS = 8, ND = 4, PB = 4;
+    constexpr unsigned TILE = 32 * DH * 2;   // 8 KiB
+    constexpr unsigned STAGE = 2 * TILE;     // K tile, V tile
+    constexpr unsigned GF0 = 2 * STAGE;      // then [4 waves][PB] d_out tiles
+    extern __shared__ __align__(16) char smem[];
+
+    const int n_qb = (T_len + 127) / 128;
+    const int n_pb = (P + PB - 1) / PB;
+    int bh, rem;
+    if (!map_block(n_qb * n_pb, n_bh, bh, rem)) return;
+    const int qb = n_qb - 1 - rem / n_pb;  // longest rows first
+    const int p0 = (rem % n_pb) * PB;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 31, h = lane >> 5;
+    const bool active = qb * 128 + wave * 32 < T_len;
+    const int i0w = min(qb * 128 + wave * 32, T_len - 32);
+    const size_t base = (size_t)bh * T_len * DH;
+    const T* k_bh = k + base;
+    const T* v_bh = v + base;
+
+    const unsigned lane_nat = m * 256 + ((h ^ swz<DH>(m)) << 4);  // ^ (ks << 5)
+    const unsigned s16 = lane & 15, g1 = (lane >> 4) & 1;
+    const unsigned lane_phys = (((s16 >> 2) & 3) << 2) | ((2 * g1 + ((s16 & 3) >> 1)) ^ h);
+    const unsigned lane_tr = (4 * h + (s16 >> 2)) * 256 + (lane_phys << 4) + ((s16 & 1) << 3);
+
+    unsigned dma_off[2];
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        const int r = 4 * (2 * wave + x) + (lane >> 4);
+        dma_off[x] = r * 256 + (((lane & 15) ^ swz<DH>(r)) << 4);
+    }
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
+    auto issue_tile = [&](int j_row, unsigned stage_base) __attribute__((always_inline)) {
+        const unsigned row_bytes = (unsigned)j_row * 256;
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            dma16(k_bh, row_bytes + dma_off[x], lds0 + stage_base + 1024 * (2 * wave + x));
+            dma16(v_bh, row_bytes + dma_off[x], lds0 + stage_base + TILE + 1024 * (2 * wave + x));
+        }
+    };
+
+    // Resident: Q fragments (B operand of S^T), lse2 and delta of the lane's query.
+    u32x4 qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+        qf[ks] = *reinterpret_cast<const u32x4*>(q + base + (size_t)(i0w + m) * DH + 16 * ks + 8 * h);
+    const float my_lse = lse2[(size_t)bh * T_len + i0w + m];
+    float my_delta[PB];
+    char* gf_w = smem + GF0 + wave * PB * TILE;
+#pragma unroll
+    for (int pp = 0; pp < PB; ++pp) {
+        const int p = min(p0 + pp, P - 1);  // surplus slots redo the last direction; never stored
+        const size_t row0 = (((size_t)b * P + p) * H + hh) * T_len + i0w;
+        my_delta[pp] = delta[row0 + m];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int slot = 64 * u + lane;
+            const int r = slot >> 4, c = slot & 15;
+            const u32x4 val = *reinterpret_cast<const u32x4*>(d_out + (row0 + r) * DH + 8 * c);
+            *reinterpret_cast<u32x4*>(gf_w + pp * TILE + tile_off<DH>(r, c)) = val;
+        }
+    }
+
+    f32x16 acc[PB][ND];
+#pragma unroll
+    for (int pp = 0; pp < PB; ++pp)
+#pragma unroll
+        for (int nd = 0; nd < ND; ++nd) acc[pp][nd] = zero16();
+    const float sc2 = scale * LOG2E;
+
+    auto tr_frag = [&](const char* tile, int kk, int nd) __attribute__((always_inline)) {
+        typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+        const s16x4 lo =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + (lane_tr ^ (nd << 6)) + (16 * kk) * 256));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_ptr)(tile + (lane_tr ^ ((nd << 6) | 32)) + (16 * kk + 8) * 256));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        return u32x4{l2[0], l2[1], h2[0], h2[1]};
+    };
+    auto nat = [&](const char* tile, int ks) __attribute__((always_inline)) {
+        return *reinterpret_cast<const u32x4*>(tile + (lane_nat ^ (ks << 5)));
+    };
+
+    // One key-tile step on the stage at byte offset SB.  thr: element 8g+e (key row) is
+    // above the diagonal for this lane's query iff 8g + e > thr.
+    auto step = [&](auto mask_tag, auto stage_tag, int thr) __attribute__((always_inline)) {
+        constexpr bool MASK = decltype(mask_tag)::value;
+        constexpr unsigned SB = decltype(stage_tag)::value;
+        const char* kt = smem + SB;
+        const char* vt = smem + SB + TILE;
+
+        // ---- S^T, all eight K fragments in flight, then the V fragments (kept for 4 directions)
+        u32x4 ka[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ka[ks] = nat(kt, ks);
+        f32x16 s = Mma<T>::mma_v_start(ka[0], qf[0]);
+#pragma unroll
+        for (int ks = 1; ks < KS; ++ks) Mma<T>::mma_v(ka[ks], qf[ks], s);
+        u32x4 va[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) va[ks] = nat(vt, ks);
+        u32x4 gfr[2];  // d_out fragment ring
+        gfr[0] = nat(gf_w, 0);
+        mma_v_settle(s);
+
+        u32x4 pq[2];           // P rounded to the storage type
+        u32x4 dsa[PB][2];      // dS_p, A operands of the dQ products
+        f32x16 dp_prev = s;    // placeholder until the first dP tile exists
+#pragma unroll
+        for (int pp = 0; pp < PB; ++pp) {
+            const char* gt = gf_w + pp * TILE;
+            f32x16 dp;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int cur = (pp * KS + ks) & 1;
+                // next fragment: same direction, or the first one of the next direction
+                if (ks + 1 < KS) gfr[cur ^ 1] = nat(gt, ks + 1);
+                else if (pp + 1 < PB) gfr[cur ^ 1] = nat(gt + TILE, 0);
+                if (ks == 0) dp = Mma<T>::mma_v_start(va[0], gfr[cur]);
+                else Mma<T>::mma_v(va[ks], gfr[cur], dp);
+                // VALU work slotted under this product: P for pp == 0, dS_{pp-1} otherwise;
+                // two (g) blocks of four elements per product for ks < 2 ... spread over ks 0..3
+                if (ks < 4) {
+                    const int g = ks;
+                    if (pp == 0) {
+                        float pr[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            pr[e] = __builtin_amdgcn_exp2f(s[4 * g + e] * sc2 - my_lse);
+                            if (MASK && (8 * g + e > thr)) pr[e] = 0.0f;
+                        }
+                        unsigned w0 = Mma<T>::pack2(pr[0], pr[1]), w1 = Mma<T>::pack2(pr[2], pr[3]);
+                        pin_here(w0, w1);
+                        pq[g >> 1][2 * (g & 1)] = w0;
+                        pq[g >> 1][2 * (g & 1) + 1] = w1;
+                    } else {
+                        const unsigned q0 = pq[g >> 1][2 * (g & 1)], q1 = pq[g >> 1][2 * (g & 1) + 1];
+                        const float dl = my_delta[pp - 1];
+                        const float d0 = Mma<T>::lo(q0) * (dp_prev[4 * g + 0] - dl);
+                        const float d1 = Mma<T>::hi(q0) * (dp_prev[4 * g + 1] - dl);
+                        const float d2 = Mma<T>::lo(q1) * (dp_prev[4 * g + 2] - dl);
+                        const float d3 = Mma<T>::hi(q1) * (dp_prev[4 * g + 3] - dl);
+                        unsigned w0 = Mma<T>::pack2(d0, d1), w1 = Mma<T>::pack2(d2, d3);
+                        pin_here(w0, w1);
+                        dsa[pp - 1][g >> 1][2 * (g & 1)] = w0;
+                        dsa[pp - 1][g >> 1][2 * (g & 1) + 1] = w1;
+                    }
+                }
+            }
+            mma_v_settle(dp);
+            dp_prev = dp;
+        }
+        // dS of the last direction, then the dQ products.
+        u32x4 kfr[2];
+        kfr[0] = tr_frag(kt, 0, 0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const unsigned q0 = pq[g >> 1][2 * (g & 1)], q1 = pq[g >> 1][2 * (g & 1) + 1];
+            const float dl = my_delta[PB - 1];
+            const float d0 = Mma<T>::lo(q0) * (dp_prev[4 * g + 0] - dl);
+            const float d1 = Mma<T>::hi(q0) * (dp_prev[4 * g + 1] - dl);
+            const float d2 = Mma<T>::lo(q1) * (dp_prev[4 * g + 2] - dl);
+            const float d3 = Mma<T>::hi(q1) * (dp_prev[4 * g + 3] - dl);
+            dsa[PB - 1][g >> 1][2 * (g & 1)] = Mma<T>::pack2(d0, d1);
+            dsa[PB - 1][g >> 1][2 * (g & 1) + 1] = Mma<T>::pack2(d2, d3);
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * ND; ++i) {
+            const int kk = i / ND, nd = i % ND, cur = i & 1;
+            if (i + 1 < 2 * ND) kfr[cur ^ 1] = tr_frag(kt, (i + 1) / ND, (i + 1) % ND);
+#pragma unroll
+            for (int pp = 0; pp < PB; ++pp) acc[pp][nd] = Mma<T>::mma(dsa[pp][kk], kfr[cur], acc[pp][nd]);
+        }
+    };
+
+    const int j_end = CAUSAL ? min(T_len, qb * 128 + 128) : T_len;
+    const int n_it = j_end / 32;                       // even
+    const int n_plain = CAUSAL ? max(0, n_it - 4) : n_it;  // steps wholly below the diagonal
+    issue_tile(0, 0);
+    auto two_steps = [&](auto mask_tag, int it) __attribute__((always_inline)) {
+        const int j0 = it * 32;
+        const int thr = i0w + m - j0 - 4 * h;
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        __syncthreads();
+        issue_tile(min(j0 + 32, T_len - 32), STAGE);
+        step(mask_tag, std::integral_constant<unsigned, 0>{}, thr);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        __syncthreads();
+        issue_tile(min(j0 + 64, T_len - 32), 0);
+        step(mask_tag, std::integral_constant<unsigned, STAGE>{}, thr - 32);
+    };
+    int it = 0;
+    for (; it < n_plain; it += 2) two_steps(std::false_type{}, it);
+    for (; it < n_it; it += 2) two_steps(std::true_type{}, it);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+
+    if (active) {
+#pragma unroll
+        for (int pp = 0; pp < PB; ++pp) {
+            if (p0 + pp >= P) break;
+            unsigned short* o =
+                reinterpret_cast<unsigned short*>(dq + ((((size_t)b * P + p0 + pp) * H + hh) * T_len + i0w) * DH);
+#pragma unroll
+            for (int nd = 0; nd < ND; ++nd)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    const unsigned two = Mma<T>::pack2(acc[pp][nd][r] * scale, acc[pp][nd][r + 1] * scale);
+                    o[(size_t)c_row(r, h) * DH + 32 * nd + m] = (unsigned short)(two & 0xffffu);
+                    o[(size_t)c_row(r + 1, h) * DH + 32 * nd + m] = (unsigned short)(two >> 16);
+                }
+        }
+    }
+}
+
+constexpr size_t dq128_lds_bytes = 2 * (2 * 32 * 128 * 2) + 4 * 4 * 32 * 128 * 2;  // K/V ring + d_out tiles
+
+template <typename T, int DH, int PB, bool CAUSAL>
+void launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
+               int H, int P, int T_len, float scale, hipStream_t stream) {
+    const int n_qb = (T_len + 127) / 128;
+    if constexpr (DH == 128) {
+        const int n_pb = (P + 3) / 4;
+        static_assert(dq128_lds_bytes <= 160 * 1024, "LDS budget");
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dq128_kernel<T, CAUSAL>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)dq128_lds_bytes);
+        hipLaunchKernelGGL((dq128_kernel<T, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), dq128_lds_bytes,
+                           stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
+    } else {
+        const int n_pb = (P + PB - 1) / PB;
+        constexpr size_t lds_bytes = 4 * 32 * DH * 2;
+        hipLaunchKernelGGL((dq_kernel<T, DH, PB, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), lds_bytes,
+                           stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
+    }
+}
+
+}  // namespace attn_mfma
+}  // namespace lbi

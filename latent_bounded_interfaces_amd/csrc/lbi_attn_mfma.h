@@ -165,6 +165,7 @@ template <typename T> __device__ __forceinline__ u32x4 pack_frag(const f32x16& c
 __device__ __forceinline__ void mma_v_settle(f32x16& c0, f32x16& c1) {
     asm volatile("s_nop 15" : "+v"(c0), "+v"(c1));
 }
+__device__ __forceinline__ void mma_v_settle(f32x16& c0) { asm volatile("s_nop 15" : "+v"(c0)); }
 
 // Pins the instructions that produce w0, w1 before this point in program order (the asm
 // MFMAs are volatile too, so VALU work written between two of them stays between them
@@ -670,6 +671,11 @@ template <typename T, int DH, bool CAUSAL>
 void launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
                  int n_bh, int H, int P, int T_len, float scale, hipStream_t stream);
 
+// dQ launch: head dim 128 has its own kernel (lbi_attn_dq128.h).
+template <typename T, int DH, int PB, bool CAUSAL>
+void launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
+               int H, int P, int T_len, float scale, hipStream_t stream);
+
 template <typename T, int DH, bool CAUSAL>
 int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T* dv, float* workspace, int B,
                  int H, int T_len, int P, float scale, hipStream_t stream) {
@@ -689,8 +695,7 @@ int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T
     constexpr int rows_per_block = 256 / (DH / 8);
     hipLaunchKernelGGL((delta_kernel<T, DH>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)),
                        dim3(256), 0, stream, g, o32, delta, H, P, T_len, n_rows);
-    hipLaunchKernelGGL((dq_kernel<T, DH, PB, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), lds_bytes,
-                       stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
+    launch_dq<T, DH, PB, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
     launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
