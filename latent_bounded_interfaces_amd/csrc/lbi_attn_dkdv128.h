@@ -6,9 +6,9 @@
 // cycles in VALU work and in waits as in MFMA.
 //
 //  * Q / d_out tiles and the lse2 / delta rows go global -> LDS with global_load_lds
-//    (16 bytes per lane, no staging registers, no ds_write), one tile ahead, into a
-//    two-stage ring.  The loop is unrolled by two so the stage is a compile-time
-//    immediate of every LDS read.
+//    (16 bytes per lane, no staging registers, no ds_write), three tiles ahead, into a
+//    four-stage ring (a tile load takes longer than a step).  The loop is unrolled by
+//    four so the stage is a compile-time immediate of every LDS read.
 //  * The XOR swizzle is linear over GF(2), so every LDS address is
 //    (lane constant) ^ (compile-time constant) + immediate: one VALU op per read at most.
 //  * Causal masking runs only in the first 8 steps of a workgroup (queries that
@@ -29,7 +29,7 @@ namespace attn_mfma {
 constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
 // 64 lanes x 16 bytes, global -> LDS.  Lane l reads 16 bytes at base + voff(l) and the
-// data lands at lds_base + 16*l.  lds_base must be wave-uniform and below 64 KiB.
+// data lands at lds_base + 16*l.  lds_base must be wave-uniform.
 __device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
@@ -48,7 +48,8 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
     constexpr unsigned STATS = 4 * 256;            // per wave: 32 lse2 + 32 delta floats
     constexpr unsigned STAGE = 2 * TILE + STATS;   // Q tile, d_out tile, stats
     constexpr int NDMA = 5;                        // global_load_lds per wave per tile
-    extern __shared__ __align__(16) char smem[];   // [2][STAGE]
+    constexpr int R = 4;                           // ring stages
+    extern __shared__ __align__(16) char smem[];   // [R][STAGE], then V
 
     const int n_kb = (T_len + 255) / 256;
     int bh, rem;
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
         for (int ks = 0; ks < KS; ++ks)
             kf[t][ks] = *reinterpret_cast<const u32x4*>(k + base + (size_t)(j0w + 32 * t + m) * DH + 16 * ks + 8 * h);
     {
-        char* vt_w = smem + 2 * STAGE + wave * 2 * TILE;
+        char* vt_w = smem + R * STAGE + wave * 2 * TILE;
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
             const int slot = 64 * u + lane;  // 16-byte slot of the wave's 64 x 256-byte block
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
             *reinterpret_cast<u32x4*>(vt_w + (r >> 5) * TILE + tile_off<DH>(r & 31, c)) = val;
         }
     }
-    const char* vt = smem + 2 * STAGE + wave * 2 * TILE;
+    const char* vt = smem + R * STAGE + wave * 2 * TILE;
     f32x16 acc_k[2][ND], acc_v[2][ND];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -241,30 +242,39 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
         }
     };
 
+    // ---- tile loop: a ring of R stages filled R-1 steps ahead.  A group is R consecutive
+    // steps, so every stage offset is an immediate.  Steps past the end of the sequence
+    // (the group count is rounded up) run on a re-read tile with everything masked.
     const int i_begin = CAUSAL ? kb * 256 : 0;
-    const int n_it = (T_len - i_begin) / 32;             // even: T_len % 64 == 0
-    const int n_mask = CAUSAL ? min(8, n_it) : 0;         // steps that can touch the diagonal
-    issue_tile(i_begin, 0);
-    // One trip = two tile steps (stage 0 then stage 1).  Before a step: this wave's share of
-    // the tile has landed (all but the newest NDMA loads done), then the barrier makes
-    // everyone's share visible and retires the other stage, which is refilled at once.
-    auto two_steps = [&](auto mask_tag, int it) __attribute__((always_inline)) {
-        const int i0 = i_begin + it * 32;
-        const int thr = j0w + m - 4 * h - i0;
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    const int n_it = (T_len - i_begin) / 32;
+    const int n_pad = (n_it + R - 1) / R * R;
+    const int head_end = CAUSAL ? min(8, n_pad) : 0;  // steps that can touch the diagonal (8 = 256 keys / 32)
+    const int plain_end = head_end + (n_it > head_end ? (n_it - head_end) / R * R : 0);
+    auto tile_row = [&](int it) __attribute__((always_inline)) { return min(i_begin + it * 32, T_len - 32); };
+#pragma unroll
+    for (int x = 0; x < R - 1; ++x) issue_tile(tile_row(x), x * STAGE);
+    auto one_step = [&](auto mask_tag, auto slot_tag, int it) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        // this wave's share of tile `it` has landed once all but the newest R-2 tile loads are done;
+        // the barrier publishes everyone's share and retires the stage read in the step before.
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((R - 2) * NDMA));
         __syncthreads();
-        issue_tile(min(i0 + 32, T_len - 32), STAGE);
-        step(mask_tag, std::integral_constant<unsigned, 0>{}, thr);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-        __syncthreads();
-        issue_tile(min(i0 + 64, T_len - 32), 0);
-        step(mask_tag, std::integral_constant<unsigned, STAGE>{}, thr - 32);
+        issue_tile(tile_row(it + R - 1), ((SLOT + R - 1) % R) * STAGE);
+        // real steps of the non-causal case mask nothing; padding steps mask everything
+        const int thr = it >= n_it ? (1 << 20) : CAUSAL ? j0w + m - 4 * h - (i_begin + it * 32) : -(1 << 20);
+        step(mask_tag, std::integral_constant<unsigned, SLOT * STAGE>{}, thr);
+    };
+    auto group = [&](auto mask_tag, int it0) __attribute__((always_inline)) {
+        one_step(mask_tag, std::integral_constant<int, 0>{}, it0);
+        one_step(mask_tag, std::integral_constant<int, 1>{}, it0 + 1);
+        one_step(mask_tag, std::integral_constant<int, 2>{}, it0 + 2);
+        one_step(mask_tag, std::integral_constant<int, 3>{}, it0 + 3);
     };
     int it = 0;
-    for (; it < n_mask; it += 2) two_steps(std::true_type{}, it);
-    for (; it < n_it; it += 2) two_steps(std::false_type{}, it);
+    for (; it < head_end; it += R) group(std::true_type{}, it);
+    for (; it < plain_end; it += R) group(std::false_type{}, it);
+    for (; it < n_pad; it += R) group(std::true_type{}, it);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-    (void)NDMA;
 
     if (active) {
         unsigned short* ok = reinterpret_cast<unsigned short*>(dk + (prow + j0w) * DH);
@@ -287,7 +297,7 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
     }
 }
 
-constexpr size_t dkdv128_lds_bytes = 2 * (2 * 32 * 128 * 2 + 4 * 256) + 4 * 2 * 32 * 128 * 2;  // stages + V
+constexpr size_t dkdv128_lds_bytes = 4 * (2 * 32 * 128 * 2 + 4 * 256) + 4 * 2 * 32 * 128 * 2;  // stages + V
 
 template <typename T, int DH, bool CAUSAL>
 void launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
