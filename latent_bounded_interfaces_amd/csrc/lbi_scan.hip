@@ -12,6 +12,8 @@
 // in a fixed order, so reruns are bit-identical.
 #include "lbi_common.h"
 
+#include <type_traits>
+
 namespace lbi {
 namespace {
 
@@ -360,6 +362,82 @@ __global__ __launch_bounds__(512) void cotangent_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Cotangent chain for d = 256, fp32: the HBM-bound case that matters.  One workgroup of
+// 8 waves per batch element; a wave takes rows wave, wave+8, ... (32 per step), one row
+// (1 KiB) per load instruction.  The matrices do not depend on the chain, so half a matrix
+// per wave is always in flight in registers (two 16-row buffers, 128 KiB per workgroup)
+// while the other half is multiplied.  The 32 partial sums of a lane are folded across
+// the 64 lanes with a halving butterfly (31 exchanges instead of 32 x 6).
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(512) void cotangent256_kernel(const float* __restrict__ mats,
+                                                           const float* __restrict__ g,
+                                                           float* __restrict__ out, int K) {
+    constexpr int D = 256;
+    __shared__ __align__(16) float vbuf[2][D];
+    const int b = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row addresses stay scalar
+    const float* mats_b = mats + (size_t)b * K * D * D;
+    float* out_b = out + (size_t)b * (K + 1) * D;
+    if (tid < D) {
+        const float val = g[(size_t)b * D + tid];
+        vbuf[0][tid] = val;
+        out_b[(size_t)K * D + tid] = val;
+    }
+    if (K == 0) return;
+    // 16 rows: wave + 8 * (16 * half + i), columns 4 * lane .. 4 * lane + 3
+    auto load_half = [&](f32x4 (&dst)[16], int r, int half) {
+        const float* base = mats_b + (size_t)r * D * D + (size_t)(wave + 128 * half) * D;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[i] = *reinterpret_cast<const f32x4*>(base + (size_t)(8 * i) * D + 4 * lane);
+    };
+    // LDS writes visible to the workgroup; loads already in flight are NOT waited for
+    // (a full __syncthreads would drain them together with the stores of the step).
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    f32x4 buf_a[16], buf_b[16];
+    load_half(buf_a, K - 1, 0);
+    lds_barrier();
+    int cur = 0;
+    for (int r = K - 1; r >= 0; --r) {
+        const f32x4 vv = *reinterpret_cast<const f32x4*>(&vbuf[cur][4 * lane]);
+        float vals[32];
+        load_half(buf_b, r, 1);
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            vals[i] = fmaf(buf_a[i][3], vv[3], fmaf(buf_a[i][2], vv[2], fmaf(buf_a[i][1], vv[1], buf_a[i][0] * vv[0])));
+        load_half(buf_a, r > 0 ? r - 1 : 0, 0);  // next step's first half (a harmless re-read at the end)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            vals[16 + i] =
+                fmaf(buf_b[i][3], vv[3], fmaf(buf_b[i][2], vv[2], fmaf(buf_b[i][1], vv[1], buf_b[i][0] * vv[0])));
+        // Halving butterfly: after the stage with mask M a lane keeps the half of its values
+        // selected by its bit M; at the end lane l holds row index l >> 1 summed over all lanes.
+        auto stage = [&](auto half_tag) {
+            constexpr int HALF = decltype(half_tag)::value;  // values kept; also the lane bit of this stage
+            const bool up = (lane & (2 * HALF)) != 0;
+            float got[HALF];
+#pragma unroll
+            for (int i = 0; i < HALF; ++i) got[i] = __shfl_xor(up ? vals[i] : vals[i + HALF], 2 * HALF, 64);
+#pragma unroll
+            for (int i = 0; i < HALF; ++i) vals[i] = (up ? vals[i + HALF] : vals[i]) + got[i];
+        };
+        stage(std::integral_constant<int, 16>{});
+        stage(std::integral_constant<int, 8>{});
+        stage(std::integral_constant<int, 4>{});
+        stage(std::integral_constant<int, 2>{});
+        stage(std::integral_constant<int, 1>{});
+        const float total = vals[0] + __shfl_xor(vals[0], 1, 64);
+        if ((lane & 1) == 0) {
+            const int row = wave + 8 * (lane >> 1);
+            vbuf[cur ^ 1][row] = total;
+            out_b[(size_t)r * D + row] = total;
+        }
+        lds_barrier();
+        cur ^= 1;
+    }
+}
+
 template <typename Tin, int D, int RT, int CB, bool COT>
 int launch_mfma_cot(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
     constexpr int NW = D / RT;
@@ -425,6 +503,12 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
     const size_t lds_bytes = (size_t)2 * dpad * sizeof(float);
     if (lds_bytes > 64 * 1024) return fail(LBI_ERR_UNSUPPORTED, "suffix cotangents: d=%d is too large (max 8192)", d);
     const int threads = d >= 128 ? 512 : (d >= 32 ? 256 : 64);
+    if (d == 256 && std::is_same<Tin, float>::value) {
+        hipLaunchKernelGGL(cotangent256_kernel, dim3(B), dim3(512), 0, stream, static_cast<const float*>(mats),
+                           static_cast<const float*>(g), static_cast<float*>(out), K);
+        LBI_HIP_CHECK(hipGetLastError());
+        return LBI_OK;
+    }
     if (d % 4 == 0)
         hipLaunchKernelGGL((cotangent_kernel<Tin, true>), dim3(B), dim3(threads), lds_bytes, stream,
                            static_cast<const Tin*>(mats), static_cast<const float*>(g),
