@@ -12,7 +12,10 @@
 // in a fixed order, so reruns are bit-identical.
 #include "lbi_common.h"
 
+#include <cstdlib>
 #include <type_traits>
+
+#include "lbi_scan_split.h"
 
 namespace lbi {
 namespace {
@@ -236,7 +239,9 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 }
             }
         }
-        __syncthreads();
+        // LDS-only barrier: the new block and v are LDS data; a full __syncthreads would also
+        // drain the mats prefetch and this step's stores.
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         cur ^= 1;
         }
     }
@@ -476,7 +481,20 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
 template <typename Tin>
 int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, int K, int d, hipStream_t stream) {
     switch (d) {
-        case 256: return launch_mfma<Tin, 256, 32, 64>(mats, out, g, cot, B, K, stream);
+        case 256: {
+            // bf16 storage runs on the 16-bit matrix pipes with exact three-way splits of the
+            // running suffix (3 bf16 products per fp32 product instead of one 16x slower fp32
+            // MFMA).  fp32 storage would need 9: measured 4 % faster than the fp32-MFMA kernel
+            // and slightly less accurate (the part clocks down under dense bf16 MFMA load), so
+            // it is opt-in: LBI_SCAN_SPLIT_FP32=1.
+            if constexpr (std::is_same<Tin, bf16_raw>::value) return scan_split::launch<Tin>(mats, out, g, cot, B, K, stream);
+            if constexpr (std::is_same<Tin, float>::value) {
+                static const bool split_fp32 =
+                    std::getenv("LBI_SCAN_SPLIT_FP32") && std::atoi(std::getenv("LBI_SCAN_SPLIT_FP32"));
+                if (split_fp32) return scan_split::launch<Tin>(mats, out, g, cot, B, K, stream);
+            }
+            return launch_mfma<Tin, 256, 32, 64>(mats, out, g, cot, B, K, stream);
+        }
         case 128: return launch_mfma<Tin, 128, 32, 32>(mats, out, g, cot, B, K, stream);
         case 64: return launch_mfma<Tin, 64, 32, 32>(mats, out, g, cot, B, K, stream);
         case 32: return launch_mfma<Tin, 32, 32, 32>(mats, out, g, cot, B, K, stream);

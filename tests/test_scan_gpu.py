@@ -211,3 +211,26 @@ def test_backward_module_contract(device):
     assert torch.allclose(one.cpu(), torch.einsum("bij,bj->bi", mats[:, 0], g), atol=1e-5, rtol=1e-5)
     stats = bs.interface_state_jacobian_t_stats(jts, include_suffix=True)
     assert {"jac_local_spec_mean", "jac_suffix_spec_max"} <= set(stats)
+
+
+def test_split_fp32_variant_in_subprocess(device):
+    """The opt-in bf16-split kernel for fp32 storage (LBI_SCAN_SPLIT_FP32=1) meets the same bar."""
+    import os
+    import subprocess
+    import sys
+
+    code = (
+        "import torch, sys; sys.path.insert(0, %r);"
+        "from oracle import scan as o;"
+        "from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks_and_cotangents as f;"
+        "m, g = o.make_scan_inputs(3, 9, 256, kind='randn', seed=5);"
+        "out, cot = f(m.cuda(), g.cuda());"
+        "t = o.suffix_scan_sequential(m, dtype=torch.float64);"
+        "e = float(((out.cpu().double() - t).abs().flatten(2).amax(2) / t.abs().flatten(2).amax(2)).max());"
+        "c = o.suffix_cotangents_sequential(m.double(), g.double());"
+        "ec = float(((cot.cpu().double() - c).abs() / c.abs().amax(2, keepdim=True)).max());"
+        "print(e, ec); sys.exit(0 if e <= 1e-5 and ec <= 1e-5 else 1)"
+    ) % str(Path(__file__).resolve().parents[1])
+    env = dict(os.environ, LBI_SCAN_SPLIT_FP32="1")
+    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stdout + res.stderr
