@@ -1,4 +1,4 @@
-// dK/dV kernel of the attention input-pullback for head dim 128 (fp16 / bf16 storage).
+// dK/dV kernel of the attention input-pullback (fp16 / bf16 storage, head dim 64 or 128).
 //
 // Same ownership and arithmetic as attn_mfma::dkdv_kernel (one wave = 64 keys x one
 // direction, workgroup = 256 keys, Q and d_out_p streamed in 32-query tiles), with the
@@ -37,17 +37,20 @@ __device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned 
                  : "memory");
 }
 
-template <typename T, bool CAUSAL>
-__global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, const T* __restrict__ k,
+template <typename T, int DH, bool CAUSAL>
+__global__ __launch_bounds__(256) void dkdv_ring_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                       const T* __restrict__ v, const T* __restrict__ d_out,
                                                       const float* __restrict__ lse2, const float* __restrict__ delta,
                                                       T* __restrict__ dk, T* __restrict__ dv, int n_bh, int H, int P,
                                                       int T_len, float scale) {
-    constexpr int DH = 128, KS = 8, ND = 4;
-    constexpr unsigned TILE = 32 * DH * 2;         // 8 KiB
+    constexpr int KS = DH / 16, ND = DH / 32;
+    constexpr int RB = DH * 2;                     // bytes per tile row
+    constexpr int CPR = DH / 8;                    // 16-byte chunks per tile row
+    constexpr int NX = DH / 64;                    // global_load_lds per tile per wave
+    constexpr unsigned TILE = 32 * RB;             // 8 KiB (Dh 128) / 4 KiB (Dh 64)
     constexpr unsigned STATS = 4 * 256;            // per wave: 32 lse2 + 32 delta floats
     constexpr unsigned STAGE = 2 * TILE + STATS;   // Q tile, d_out tile, stats
-    constexpr int NDMA = 5;                        // global_load_lds per wave per tile
+    constexpr int NDMA = 2 * NX + 1;               // global_load_lds per wave per tile step
     constexpr int R = 4;                           // ring stages
     extern __shared__ __align__(16) char smem[];   // [R][STAGE], then V
 
@@ -68,30 +71,34 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
     const float* delta_p = delta + prow;
 
     // ---- lane constants of the LDS addressing -------------------------------------------
-    const unsigned lane_nat = m * 256 + ((h ^ swz<DH>(m)) << 4);  // ^ (ks << 5)
+    // nat: tile_off(m, 2ks + h) == lane_nat ^ (ks << 5).  tr: the address of the transpose read for
+    // (k0, hi, nd) is (lane_tr ^ (nd << 6 | hi << 5)) + (k0 + 8 hi) * RB; both follow from the
+    // swizzle being an XOR of row bits into chunk bits.
+    const unsigned lane_nat = m * RB + ((h ^ swz<DH>(m)) << 4);
     const unsigned s16 = lane & 15, g1 = (lane >> 4) & 1;
-    const unsigned lane_phys = (((s16 >> 2) & 3) << 2) | ((2 * g1 + ((s16 & 3) >> 1)) ^ h);
-    const unsigned lane_tr = (4 * h + (s16 >> 2)) * 256 + (lane_phys << 4) + ((s16 & 1) << 3);  // ^ (nd<<6 | hi<<5)
+    const unsigned tr_row = 4 * h + (s16 >> 2), tr_chunk = 2 * g1 + ((s16 & 3) >> 1);
+    const unsigned lane_tr = tr_row * RB + ((tr_chunk ^ swz<DH>(tr_row)) << 4) + ((s16 & 1) << 3);
     const unsigned lane_stat = (unsigned)wave * 256 + 16 * h;  // + 32*g (lse2), + 128 (delta)
 
     // ---- global -> LDS: this wave's share of a tile step ---------------------------------
-    // Tile slot sigma = 64u + lane (u = 2*wave, 2*wave+1): row sigma/16, physical chunk sigma%16.
-    unsigned dma_off[2];
+    // Tile slot sigma = 64u + lane (u = NX*wave + x): row sigma/CPR, physical chunk sigma%CPR.
+    unsigned dma_off[NX];
 #pragma unroll
-    for (int x = 0; x < 2; ++x) {
-        const int r = 4 * (2 * wave + x) + (lane >> 4);
-        dma_off[x] = r * 256 + (((lane & 15) ^ swz<DH>(r)) << 4);
+    for (int x = 0; x < NX; ++x) {
+        const int sigma = 64 * (NX * wave + x) + lane;
+        const int r = sigma / CPR;
+        dma_off[x] = r * RB + (((sigma % CPR) ^ swz<DH>(r)) << 4);
     }
     // lanes 0-7: lse2 float4 #lane, lanes 8-15: delta float4 #(lane-8), as offsets from lse_bh
     const unsigned stat_off =
         (lane < 8 ? 0u : (unsigned)((const char*)delta_p - (const char*)lse_bh)) + 16 * (lane & 7);
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
     auto issue_tile = [&](int i_row, unsigned stage_base) __attribute__((always_inline)) {
-        const unsigned row_bytes = (unsigned)i_row * 256;
+        const unsigned row_bytes = (unsigned)i_row * RB;
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            dma16(q_bh, row_bytes + dma_off[x], lds0 + stage_base + 1024 * (2 * wave + x));
-            dma16(g_p, row_bytes + dma_off[x], lds0 + stage_base + TILE + 1024 * (2 * wave + x));
+        for (int x = 0; x < NX; ++x) {
+            dma16(q_bh, row_bytes + dma_off[x], lds0 + stage_base + 1024 * (NX * wave + x));
+            dma16(g_p, row_bytes + dma_off[x], lds0 + stage_base + TILE + 1024 * (NX * wave + x));
         }
         // Every wave keeps its own copy of the 64 row statistics: no cross-wave dependency.
         if (lane < 16) dma16(lse_bh, (unsigned)i_row * 4 + stat_off, lds0 + stage_base + 2 * TILE + 256 * wave);
@@ -109,9 +116,9 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
     {
         char* vt_w = smem + R * STAGE + wave * 2 * TILE;
 #pragma unroll
-        for (int u = 0; u < 16; ++u) {
-            const int slot = 64 * u + lane;  // 16-byte slot of the wave's 64 x 256-byte block
-            const int r = slot >> 4, c = slot & 15;
+        for (int u = 0; u < CPR; ++u) {
+            const int slot = 64 * u + lane;  // 16-byte slot of the wave's 64-row block
+            const int r = slot / CPR, c = slot % CPR;
             const u32x4 val = *reinterpret_cast<const u32x4*>(v + base + (size_t)(j0w + r) * DH + 8 * c);
             *reinterpret_cast<u32x4*>(vt_w + (r >> 5) * TILE + tile_off<DH>(r & 31, c)) = val;
         }
@@ -140,9 +147,9 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
     auto tr_frag = [&](const char* tile, int kk, int nd) __attribute__((always_inline)) {
         typedef __attribute__((address_space(3))) s16x4* lds_ptr;
         const s16x4 lo =
-            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + (lane_tr ^ (nd << 6)) + (16 * kk) * 256));
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + (lane_tr ^ (nd << 6)) + (16 * kk) * RB));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_ptr)(tile + (lane_tr ^ ((nd << 6) | 32)) + (16 * kk + 8) * 256));
+            (lds_ptr)(tile + (lane_tr ^ ((nd << 6) | 32)) + (16 * kk + 8) * RB));
         const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
         return u32x4{l2[0], l2[1], h2[0], h2[1]};
     };
@@ -194,18 +201,22 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
                 Mma<T>::mma_v(ga[cur], va[cur], dp[0]);
                 Mma<T>::mma_v(ga[cur], vb[cur], dp[1]);
             }
-            const int g = ks >> 1, t = ks & 1;
-            float pr[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                pr[e] = __builtin_amdgcn_exp2f(s[t][4 * g + e] * sc2 - l4[e]);
-                if (MASK && (8 * g + e < thr + 32 * t)) pr[e] = 0.0f;
+            for (int bb = 0; bb < 8 / KS; ++bb) {  // the eight (g, t) blocks of S spread over the KS products
+                const int blk = ks * (8 / KS) + bb;
+                const int g = blk >> 1, t = blk & 1;
+                float pr[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    pr[e] = __builtin_amdgcn_exp2f(s[t][4 * g + e] * sc2 - l4[e]);
+                    if (MASK && (8 * g + e < thr + 32 * t)) pr[e] = 0.0f;
+                }
+                unsigned w0 = Mma<T>::pack2(pr[0], pr[1]), w1 = Mma<T>::pack2(pr[2], pr[3]);
+                if (t == 1 && g < 3) l4 = lds_f4(st + lane_stat + 32 * (g + 1));
+                pin_here(w0, w1);
+                pa[t][g >> 1][2 * (g & 1)] = w0;
+                pa[t][g >> 1][2 * (g & 1) + 1] = w1;
             }
-            unsigned w0 = Mma<T>::pack2(pr[0], pr[1]), w1 = Mma<T>::pack2(pr[2], pr[3]);
-            if (t == 1 && g < 3) l4 = lds_f4(st + lane_stat + 32 * (g + 1));
-            pin_here(w0, w1);
-            pa[t][g >> 1][2 * (g & 1)] = w0;
-            pa[t][g >> 1][2 * (g & 1) + 1] = w1;
         }
         f32x4 d4 = lds_f4(st + lane_stat + 128);
         u32x4 bfr[2];  // tr fragments of step i live in slot i & 1
@@ -219,17 +230,21 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
             bfr[cur ^ 1] = (i + 1 < 2 * ND) ? tr_frag(gt, (i + 1) / ND, (i + 1) % ND) : tr_frag(qt, 0, 0);
             acc_v[0][nd] = Mma<T>::mma(pa[0][kk], bfr[cur], acc_v[0][nd]);
             acc_v[1][nd] = Mma<T>::mma(pa[1][kk], bfr[cur], acc_v[1][nd]);
-            const int g = i >> 1, t = i & 1;
-            const unsigned p0 = pa[t][g >> 1][2 * (g & 1)], p1 = pa[t][g >> 1][2 * (g & 1) + 1];
-            const float d0 = Mma<T>::lo(p0) * (dp[t][4 * g + 0] - d4[0]);
-            const float d1 = Mma<T>::hi(p0) * (dp[t][4 * g + 1] - d4[1]);
-            const float d2 = Mma<T>::lo(p1) * (dp[t][4 * g + 2] - d4[2]);
-            const float d3 = Mma<T>::hi(p1) * (dp[t][4 * g + 3] - d4[3]);
-            unsigned w0 = Mma<T>::pack2(d0, d1), w1 = Mma<T>::pack2(d2, d3);
-            if (t == 1 && g < 3) d4 = lds_f4(st + lane_stat + 128 + 32 * (g + 1));
-            pin_here(w0, w1);
-            dsa[t][g >> 1][2 * (g & 1)] = w0;
-            dsa[t][g >> 1][2 * (g & 1) + 1] = w1;
+#pragma unroll
+            for (int bb = 0; bb < 4 / ND; ++bb) {  // the eight (g, t) blocks of dS spread over the 2 ND steps
+                const int blk = i * (4 / ND) + bb;
+                const int g = blk >> 1, t = blk & 1;
+                const unsigned p0 = pa[t][g >> 1][2 * (g & 1)], p1 = pa[t][g >> 1][2 * (g & 1) + 1];
+                const float d0 = Mma<T>::lo(p0) * (dp[t][4 * g + 0] - d4[0]);
+                const float d1 = Mma<T>::hi(p0) * (dp[t][4 * g + 1] - d4[1]);
+                const float d2 = Mma<T>::lo(p1) * (dp[t][4 * g + 2] - d4[2]);
+                const float d3 = Mma<T>::hi(p1) * (dp[t][4 * g + 3] - d4[3]);
+                unsigned w0 = Mma<T>::pack2(d0, d1), w1 = Mma<T>::pack2(d2, d3);
+                if (t == 1 && g < 3) d4 = lds_f4(st + lane_stat + 128 + 32 * (g + 1));
+                pin_here(w0, w1);
+                dsa[t][g >> 1][2 * (g & 1)] = w0;
+                dsa[t][g >> 1][2 * (g & 1) + 1] = w1;
+            }
         }
 
         // ---- dK += dS^T Q
@@ -297,23 +312,20 @@ __global__ __launch_bounds__(256) void dkdv128_kernel(const T* __restrict__ q, c
     }
 }
 
-constexpr size_t dkdv128_lds_bytes = 4 * (2 * 32 * 128 * 2 + 4 * 256) + 4 * 2 * 32 * 128 * 2;  // stages + V
+template <int DH> constexpr size_t dkdv_ring_lds_bytes() {
+    return 4 * (2 * 32 * DH * 2 + 4 * 256) + 4 * 2 * 32 * DH * 2;  // 4 stages + V of 256 keys
+}
 
 template <typename T, int DH, bool CAUSAL>
 void launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
                  int n_bh, int H, int P, int T_len, float scale, hipStream_t stream) {
     const int n_kb = (T_len + 255) / 256;
-    if constexpr (DH == 128) {
-        static_assert(dkdv128_lds_bytes <= 160 * 1024, "LDS budget");
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dkdv128_kernel<T, CAUSAL>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkdv128_lds_bytes);
-        hipLaunchKernelGGL((dkdv128_kernel<T, CAUSAL>), dim3(grid_size(n_kb * P, n_bh)), dim3(256), dkdv128_lds_bytes,
-                           stream, q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale);
-    } else {
-        constexpr size_t lds_bytes = 4 * 32 * DH * 2 + 2 * 64 * sizeof(float);
-        hipLaunchKernelGGL((dkdv_kernel<T, DH, CAUSAL>), dim3(grid_size(n_kb * P, n_bh)), dim3(256), lds_bytes, stream,
-                           q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale);
-    }
+    constexpr size_t lds_bytes = dkdv_ring_lds_bytes<DH>();
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dkdv_ring_kernel<T, DH, CAUSAL>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipLaunchKernelGGL((dkdv_ring_kernel<T, DH, CAUSAL>), dim3(grid_size(n_kb * P, n_bh)), dim3(256), lds_bytes, stream,
+                       q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale);
 }
 
 }  // namespace attn_mfma

@@ -1,7 +1,8 @@
-// dQ kernel of the attention input-pullback for head dim 128 (fp16 / bf16 storage).
+// dQ kernel of the attention input-pullback (fp16 / bf16 storage, head dim 64 or 128).
 //
-// One wave owns 32 queries and PB = 4 directions (the 256 accumulation registers are
-// exactly its four dQ tiles of 32 x 128); a workgroup is 4 waves = 128 queries.
+// One wave owns 32 queries and PB directions (at head dim 128 the 256 accumulation registers
+// are exactly its four dQ tiles of 32 x 128; head dim 64 has room for eight); a workgroup is
+// 4 waves = 128 queries.
 //   S^T  = K Q^T        A = K tile (LDS, shared), B = Q (registers)   lanes = queries, registers = keys
 //   P    = exp2(S^T c - lse2), once for the four directions
 //   dP^T = V dO_p^T     A = V tile (LDS, shared), B = dO_p (LDS, private to the wave)
@@ -19,14 +20,18 @@
 namespace lbi {
 namespace attn_mfma {
 
-template <typename T, bool CAUSAL>
-__global__ __launch_bounds__(256) void dq128_kernel(const T* __restrict__ q, const T* __restrict__ k,
+template <typename T, int DH, int PB, bool CAUSAL>
+__global__ __launch_bounds__(256) void dq_ring_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                     const T* __restrict__ v, const T* __restrict__ d_out,
                                                     const float* __restrict__ lse2, const float* __restrict__ delta,
                                                     T* __restrict__ dq, int n_bh, int H, int P, int T_len,
                                                     float scale) {
-    constexpr int DH = 128, KS = 8, ND = 4, PB = 4;
-    constexpr unsigned TILE = 32 * DH * 2;   // 8 KiB
+    constexpr int KS = DH / 16, ND = DH / 32;
+    constexpr int RB = DH * 2;               // bytes per tile row
+    constexpr int CPR = DH / 8;              // 16-byte chunks per tile row
+    constexpr int NX = DH / 64;              // global_load_lds per tile per wave
+    static_assert(KS >= 4 && PB * ND <= 16, "four VALU blocks per direction; 256 accumulation registers");
+    constexpr unsigned TILE = 32 * RB;       // 8 KiB (Dh 128) / 4 KiB (Dh 64)
     constexpr unsigned STAGE = 2 * TILE;     // K tile, V tile
     constexpr unsigned GF0 = 2 * STAGE;      // then [4 waves][PB] d_out tiles
     extern __shared__ __align__(16) char smem[];
@@ -45,24 +50,25 @@ __global__ __launch_bounds__(256) void dq128_kernel(const T* __restrict__ q, con
     const T* k_bh = k + base;
     const T* v_bh = v + base;
 
-    const unsigned lane_nat = m * 256 + ((h ^ swz<DH>(m)) << 4);  // ^ (ks << 5)
+    const unsigned lane_nat = m * RB + ((h ^ swz<DH>(m)) << 4);  // ^ (ks << 5)
     const unsigned s16 = lane & 15, g1 = (lane >> 4) & 1;
-    const unsigned lane_phys = (((s16 >> 2) & 3) << 2) | ((2 * g1 + ((s16 & 3) >> 1)) ^ h);
-    const unsigned lane_tr = (4 * h + (s16 >> 2)) * 256 + (lane_phys << 4) + ((s16 & 1) << 3);
+    const unsigned tr_row = 4 * h + (s16 >> 2), tr_chunk = 2 * g1 + ((s16 & 3) >> 1);
+    const unsigned lane_tr = tr_row * RB + ((tr_chunk ^ swz<DH>(tr_row)) << 4) + ((s16 & 1) << 3);
 
-    unsigned dma_off[2];
+    unsigned dma_off[NX];
 #pragma unroll
-    for (int x = 0; x < 2; ++x) {
-        const int r = 4 * (2 * wave + x) + (lane >> 4);
-        dma_off[x] = r * 256 + (((lane & 15) ^ swz<DH>(r)) << 4);
+    for (int x = 0; x < NX; ++x) {
+        const int sigma = 64 * (NX * wave + x) + lane;
+        const int r = sigma / CPR;
+        dma_off[x] = r * RB + (((sigma % CPR) ^ swz<DH>(r)) << 4);
     }
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
     auto issue_tile = [&](int j_row, unsigned stage_base) __attribute__((always_inline)) {
-        const unsigned row_bytes = (unsigned)j_row * 256;
+        const unsigned row_bytes = (unsigned)j_row * RB;
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            dma16(k_bh, row_bytes + dma_off[x], lds0 + stage_base + 1024 * (2 * wave + x));
-            dma16(v_bh, row_bytes + dma_off[x], lds0 + stage_base + TILE + 1024 * (2 * wave + x));
+        for (int x = 0; x < NX; ++x) {
+            dma16(k_bh, row_bytes + dma_off[x], lds0 + stage_base + 1024 * (NX * wave + x));
+            dma16(v_bh, row_bytes + dma_off[x], lds0 + stage_base + TILE + 1024 * (NX * wave + x));
         }
     };
 
@@ -80,9 +86,9 @@ __global__ __launch_bounds__(256) void dq128_kernel(const T* __restrict__ q, con
         const size_t row0 = (((size_t)b * P + p) * H + hh) * T_len + i0w;
         my_delta[pp] = delta[row0 + m];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < CPR / 2; ++u) {
             const int slot = 64 * u + lane;
-            const int r = slot >> 4, c = slot & 15;
+            const int r = slot / CPR, c = slot % CPR;
             const u32x4 val = *reinterpret_cast<const u32x4*>(d_out + (row0 + r) * DH + 8 * c);
             *reinterpret_cast<u32x4*>(gf_w + pp * TILE + tile_off<DH>(r, c)) = val;
         }
@@ -98,9 +104,9 @@ __global__ __launch_bounds__(256) void dq128_kernel(const T* __restrict__ q, con
     auto tr_frag = [&](const char* tile, int kk, int nd) __attribute__((always_inline)) {
         typedef __attribute__((address_space(3))) s16x4* lds_ptr;
         const s16x4 lo =
-            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + (lane_tr ^ (nd << 6)) + (16 * kk) * 256));
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + (lane_tr ^ (nd << 6)) + (16 * kk) * RB));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_ptr)(tile + (lane_tr ^ ((nd << 6) | 32)) + (16 * kk + 8) * 256));
+            (lds_ptr)(tile + (lane_tr ^ ((nd << 6) | 32)) + (16 * kk + 8) * RB));
         const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
         return u32x4{l2[0], l2[1], h2[0], h2[1]};
     };
@@ -239,25 +245,24 @@ __global__ __launch_bounds__(256) void dq128_kernel(const T* __restrict__ q, con
     }
 }
 
-constexpr size_t dq128_lds_bytes = 2 * (2 * 32 * 128 * 2) + 4 * 4 * 32 * 128 * 2;  // K/V ring + d_out tiles
+template <int DH, int PB> constexpr size_t dq_ring_lds_bytes() {
+    return 2 * (2 * 32 * DH * 2) + 4 * PB * 32 * DH * 2;  // K/V ring + d_out tiles of four waves
+}
 
+// PB is the direction block of the caller's choice for head dim 64 (4 or 8); head dim 128 has
+// accumulation registers for four.
 template <typename T, int DH, int PB, bool CAUSAL>
 void launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
                int H, int P, int T_len, float scale, hipStream_t stream) {
+    constexpr int PBK = DH == 128 ? 4 : PB;
     const int n_qb = (T_len + 127) / 128;
-    if constexpr (DH == 128) {
-        const int n_pb = (P + 3) / 4;
-        static_assert(dq128_lds_bytes <= 160 * 1024, "LDS budget");
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dq128_kernel<T, CAUSAL>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)dq128_lds_bytes);
-        hipLaunchKernelGGL((dq128_kernel<T, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), dq128_lds_bytes,
-                           stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
-    } else {
-        const int n_pb = (P + PB - 1) / PB;
-        constexpr size_t lds_bytes = 4 * 32 * DH * 2;
-        hipLaunchKernelGGL((dq_kernel<T, DH, PB, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), lds_bytes,
-                           stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
-    }
+    const int n_pb = (P + PBK - 1) / PBK;
+    constexpr size_t lds_bytes = dq_ring_lds_bytes<DH, PBK>();
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dq_ring_kernel<T, DH, PBK, CAUSAL>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipLaunchKernelGGL((dq_ring_kernel<T, DH, PBK, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), lds_bytes,
+                       stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
 }
 
 }  // namespace attn_mfma
