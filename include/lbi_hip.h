@@ -118,6 +118,80 @@ int lbi_attn_pullback(const void* q, const void* k, const void* v, const void* d
                       int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P,
                       float softmax_scale, int causal, int dtype, void* stream);
 
+/*
+ * Region-level input pullback of a Transformer block (the pieces around the matrix products,
+ * which the caller issues as plain GEMMs, and around lbi_attn_pullback).  Together they
+ * implement TransformerLowering.input_pullback_basis of the reference
+ * (backends/transformer.py:64-75; stub backends/transformer_cuda.py:45-64) for the block
+ * of backends/transformer.py:118-215.  Cotangent tensors carry a basis axis: [B, P, T, *];
+ * forward activations are [B, T, *] and are shared by the P directions.
+ */
+
+/*
+ * RMSNorm pullback, optionally fused with the residual-stream add.
+ *
+ *   y = (x_r * rsqrt(mean(x_r^2) + eps)) * weight,   x_r = x rounded to branch_dtype
+ *   g_x = r * (weight o g_out) - x_r * r^3 * mean(x_r o weight o g_out)
+ *   out = g_x + g_residual            (g_residual may be NULL = 0)
+ *
+ *   g_out [B,P,T,D] and weight [D] in branch_dtype; x [B,T,D] in x_dtype (the pre-norm
+ *   residual stream, reference backends/transformer.py:197,201);
+ *   g_residual [B,P,T,D] fp32 or NULL; outputs g_sum [B,P,T,D] fp32 and/or g_sum_branch
+ *   [B,P,T,D] branch_dtype (either may be NULL, not both).  g_sum may alias g_residual.
+ *   Forward: RMSNorm.forward, reference backbones/transformer/block.py:12-23, applied by
+ *   TransformerBlock._prenorm (block.py:66-76).
+ */
+int lbi_rmsnorm_pullback(const void* g_out, const void* x, const void* weight, const void* g_residual,
+                         void* g_sum, void* g_sum_branch,
+                         int64_t B, int64_t P, int64_t T, int64_t D, float eps,
+                         int branch_dtype, int x_dtype, void* stream);
+
+/*
+ * Gated-MLP pullback through  down_input = up * silu(gate),  [up | gate] = fc1_output.
+ *
+ *   g_down_input [B,P,T,hidden], fc1_output [B,T,2*hidden]  ->  g_fc1_output [B,P,T,2*hidden]
+ *   g_up = g * silu(gate);   g_gate = g * up * silu'(gate)
+ *
+ * Forward: reference backends/transformer.py:172-176 (GatedMLP.forward,
+ * backbones/transformer/mlp.py:30-32).
+ */
+int lbi_gated_mlp_pullback(const void* g_down_input, const void* fc1_output, void* g_fc1_output,
+                           int64_t B, int64_t P, int64_t T, int64_t hidden, int dtype, void* stream);
+
+/*
+ * Head split of the out_proj-input cotangent: [B,P,T,H*Dh] -> [B,P,H,T,Dh], the layout
+ * lbi_attn_pullback takes as d_out (transpose of reference backends/transformer.py:152-153).
+ */
+int lbi_attn_heads_split(const void* g_merged, void* g_heads,
+                         int64_t B, int64_t P, int64_t T, int64_t H, int64_t Dh, int dtype, void* stream);
+
+/*
+ * Cotangent of the packed q/k/v projection from the outputs of lbi_attn_pullback.
+ *
+ *   dq, dk, dv [B,P,H,T,Dh]  ->  g_qkv [B,P,T,(H + 2*Hkv)*Dh]
+ *   q part: transposed rotary embedding of dq;  k part: the same of the sum of dk over the
+ *   H/Hkv query heads that share a key head;  v part: that sum of dv.
+ *   rope_cos, rope_sin [T, Dh/2] fp32: cos and sin of position * base^(-2i/Dh).
+ *
+ * Transposes reference backends/transformer.py:124-132 (split, head views, apply_rope of
+ * backbones/transformer/rope.py:6-34 in its half-split or interleaved pairing, and
+ * CausalSelfAttention._expand_kv, backbones/transformer/attention.py:61-65).
+ */
+int lbi_attn_qkv_pullback(const void* dq, const void* dk, const void* dv,
+                          const float* rope_cos, const float* rope_sin, void* g_qkv,
+                          int64_t B, int64_t P, int64_t T, int64_t H, int64_t Hkv, int64_t Dh,
+                          int interleaved, int dtype, void* stream);
+
+/*
+ * Pullback of the depthwise causal convolution applied to the packed projection
+ * (reference backends/transformer.py:121-122: Conv1d(groups=C, padding=k-1), first T outputs).
+ *
+ *   g_out [N,T,C], weight [C,k]  ->  g_in [N,T,C],   N = B*P
+ *   g_in[n,s,c] = sum_i weight[c,k-1-i] * g_out[n,s+i,c]   over s+i < T
+ */
+int lbi_causal_conv1d_pullback(const void* g_out, const void* weight, void* g_in,
+                               int64_t N, int64_t T, int64_t C, int64_t ksize, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,6 +11,7 @@ from typing import Any
 import torch
 
 from ..hip.transformer import attention_input_pullback_basis as hip_attention_input_pullback_basis
+from ..hip.transformer.region import region_input_pullback_basis
 
 
 class HipTransformerLowering:
@@ -19,9 +20,10 @@ class HipTransformerLowering:
     name = "hip"
 
     def __init__(self, *, reference_lowering: Any | None = None) -> None:
-        # The reference's class can delegate the two region-level methods to its autograd
-        # lowering (allow_reference_fallback=True).  Here a caller may pass any object that
-        # implements them; without one they raise, as the reference does by default.
+        # The reference's class can delegate the region-level methods to its autograd lowering
+        # (allow_reference_fallback=True).  Here input_pullback_basis always runs the HIP path;
+        # parameter_vjp is delegated to `reference_lowering` when one is given and raises
+        # otherwise, as the reference does by default.
         self.reference_lowering = reference_lowering
         self.allow_reference_fallback = reference_lowering is not None
 
@@ -49,18 +51,17 @@ class HipTransformerLowering:
         )
 
     def input_pullback_basis(self, *, backend: Any, cache: Any, output_cotangent_basis: torch.Tensor) -> torch.Tensor:
-        # reference backends/transformer_cuda.py:45-64
+        """Region input pullback ``[B, P, T, D] -> [B, P, T, D]`` on the GPU.
+
+        The method the reference leaves as the "CUDA kernel target"
+        (backends/transformer_cuda.py:45-64); same result as its autograd lowering
+        (backends/transformer.py:284-330).  ``backend`` and ``cache`` are the reference's
+        ``TransformerRegionBackend`` and ``TransformerRegionCache`` (or objects with the same
+        attribute names).
+        """
         if output_cotangent_basis.dim() != 4:
             raise ValueError("output_cotangent_basis must have shape [B, P, T, D]")
-        if self.reference_lowering is not None:
-            return self.reference_lowering.input_pullback_basis(
-                backend=backend, cache=cache, output_cotangent_basis=output_cotangent_basis
-            )
-        raise NotImplementedError(
-            "HipTransformerLowering.input_pullback_basis: the region-level input pullback for "
-            "output_cotangent_basis [B, P, T, D] is not implemented; pass reference_lowering=... "
-            "to delegate it."
-        )
+        return region_input_pullback_basis(backend, cache, output_cotangent_basis, kernel_mode="hip")
 
     def parameter_vjp(self, *, backend: Any, cache: Any, output_cotangent: torch.Tensor) -> dict[str, torch.Tensor]:
         # reference backends/transformer_cuda.py:66-83

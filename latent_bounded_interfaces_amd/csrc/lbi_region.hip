@@ -1,0 +1,515 @@
+// Region-level input pullback of a Transformer block: the memory-bound pieces between the
+// matrix products (which the host issues as library GEMMs) and the attention pullback.
+//
+// A cotangent basis carries P directions, so every tensor here is [B, P, T, *] while the
+// forward activations it is combined with are [B, T, *]: each kernel reads the activation
+// row of (b, t) for all P directions of that token and never materialises a broadcast copy.
+// All arithmetic is fp32; 16-bit storage is rounded to nearest-even on the way out.
+//
+//   rmsnorm_pullback      g_x = r (w o g_y) - x r^3 mean(x o w o g_y)  (+ residual cotangent)
+//   gated_mlp_pullback    (up, gate) cotangents of  up * silu(gate)
+//   heads_split           [B,P,T,H,Dh] -> [B,P,H,T,Dh]
+//   qkv_pullback          dq, dk, dv [B,P,H,T,Dh] -> cotangent of the packed projection
+//                         [B,P,T,(H+2Hkv) Dh]: sum over the query heads of a KV group,
+//                         transposed rotary embedding, head merge
+//   causal_conv1d_pullback  transpose of the depthwise causal convolution over T
+#include <hip/hip_runtime.h>
+
+#include "lbi_common.h"
+
+namespace lbi {
+namespace region {
+
+template <typename T> __device__ __forceinline__ T from_f32(float x);
+template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
+template <> __device__ __forceinline__ _Float16 from_f32<_Float16>(float x) { return (_Float16)x; }
+template <> __device__ __forceinline__ bf16_raw from_f32<bf16_raw>(float x) { return bf16_raw{f32_to_bf16_bits(x)}; }
+
+// x rounded to storage type T and widened again (the value a T-typed tensor would hold).
+template <typename T> __device__ __forceinline__ float round_via(float x) { return to_f32(from_f32<T>(x)); }
+
+template <typename T, int VEC> struct Pack;
+template <typename T> struct Pack<T, 1> {
+    float v[1];
+    __device__ __forceinline__ void load(const T* p) { v[0] = to_f32(p[0]); }
+    __device__ __forceinline__ void store(T* p) const { p[0] = from_f32<T>(v[0]); }
+};
+template <typename T> struct Pack<T, 4> {
+    float v[4];
+    __device__ __forceinline__ void load(const T* p) {
+        const f32x4 t = load4(p);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = t[i];
+    }
+    __device__ __forceinline__ void store(T* p) const;
+};
+template <> __device__ __forceinline__ void Pack<float, 4>::store(float* p) const {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+}
+template <> __device__ __forceinline__ void Pack<_Float16, 4>::store(_Float16* p) const {
+    *reinterpret_cast<f16x4*>(p) = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+}
+template <> __device__ __forceinline__ void Pack<bf16_raw, 4>::store(bf16_raw* p) const {
+    *reinterpret_cast<u16x4*>(p) =
+        u16x4{f32_to_bf16_bits(v[0]), f32_to_bf16_bits(v[1]), f32_to_bf16_bits(v[2]), f32_to_bf16_bits(v[3])};
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
+    return x;
+}
+
+// ---------------------------------------------------------------------------------------
+// RMSNorm pullback.  One wave per cotangent row (b, p, t); the row is read twice (sums,
+// then outputs), the second time from cache.  x is first rounded to the storage type the
+// norm ran in (TB), as the forward does.
+// ---------------------------------------------------------------------------------------
+template <typename TB, typename TX, int VEC>
+__global__ __launch_bounds__(256) void rmsnorm_pullback_kernel(const TB* __restrict__ g_out, const TX* __restrict__ x,
+                                                               const TB* __restrict__ weight,
+                                                               const float* g_residual, float* g_sum,
+                                                               TB* __restrict__ g_sum_branch, long long n_rows,
+                                                               int P, int T_len, int D, float eps) {
+    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    const long long bp = row / T_len;
+    const int t = (int)(row - bp * T_len);
+    const long long b = bp / P;
+    const TB* g_row = g_out + row * D;
+    const TX* x_row = x + (b * T_len + t) * D;
+
+    float ss = 0.0f, dot = 0.0f;
+    for (int j = lane * VEC; j < D; j += 64 * VEC) {
+        Pack<TB, VEC> g, w;
+        Pack<TX, VEC> xv;
+        g.load(g_row + j);
+        w.load(weight + j);
+        xv.load(x_row + j);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const float xr = round_via<TB>(xv.v[i]);
+            ss = fmaf(xr, xr, ss);
+            dot = fmaf(xr, w.v[i] * g.v[i], dot);
+        }
+    }
+    ss = wave_sum(ss);
+    dot = wave_sum(dot);
+    const float r = rsqrtf(ss / (float)D + eps);
+    const float c = r * r * r * dot / (float)D;
+    for (int j = lane * VEC; j < D; j += 64 * VEC) {
+        Pack<TB, VEC> g, w, ob;
+        Pack<TX, VEC> xv;
+        Pack<float, VEC> res, of;
+        g.load(g_row + j);
+        w.load(weight + j);
+        xv.load(x_row + j);
+        if (g_residual != nullptr) res.load(g_residual + row * D + j);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const float xr = round_via<TB>(xv.v[i]);
+            float o = r * (w.v[i] * g.v[i]) - xr * c;
+            if (g_residual != nullptr) o += res.v[i];
+            of.v[i] = o;
+            ob.v[i] = o;
+        }
+        if (g_sum != nullptr) of.store(g_sum + row * D + j);
+        if (g_sum_branch != nullptr) ob.store(g_sum_branch + row * D + j);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Gated MLP pullback.  fc1_output rows are [up | gate]; the forward computed
+// down_input = up * silu(gate) with silu(gate) rounded to the storage type.
+// ---------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gated_mlp_pullback_kernel(const T* __restrict__ g_down_input,
+                                                                 const T* __restrict__ fc1_output,
+                                                                 T* __restrict__ g_fc1_output, long long n_units, int P,
+                                                                 int T_len, int hidden) {
+    const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (unit >= n_units) return;
+    const int per_row = hidden / VEC;
+    const long long row = unit / per_row;
+    const int j = (int)(unit - row * per_row) * VEC;
+    const long long bp = row / T_len;
+    const int t = (int)(row - bp * T_len);
+    const long long act_row = (bp / P) * T_len + t;
+    Pack<T, VEC> g, up, gate, o_up, o_gate;
+    g.load(g_down_input + row * hidden + j);
+    up.load(fc1_output + act_row * 2 * hidden + j);
+    gate.load(fc1_output + act_row * 2 * hidden + hidden + j);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        const float z = gate.v[i];
+        const float sig = 1.0f / (1.0f + __expf(-z));
+        const float act = round_via<T>(z * sig);
+        o_up.v[i] = g.v[i] * act;
+        o_gate.v[i] = round_via<T>(g.v[i] * up.v[i]) * (sig * (1.0f + z * (1.0f - sig)));
+    }
+    o_up.store(g_fc1_output + row * 2 * hidden + j);
+    o_gate.store(g_fc1_output + row * 2 * hidden + hidden + j);
+}
+
+// ---------------------------------------------------------------------------------------
+// Head split: in [N, T, H, Dh] -> out [N, H, T, Dh]  (N = B * P), 16-byte chunks when Dh allows.
+// ---------------------------------------------------------------------------------------
+template <typename CHUNK>
+__global__ __launch_bounds__(256) void heads_split_kernel(const CHUNK* __restrict__ in, CHUNK* __restrict__ out,
+                                                          long long n_chunks, int T_len, int H, int chunks_per_head) {
+    const long long o = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (o >= n_chunks) return;
+    const int c = (int)(o % chunks_per_head);
+    long long rest = o / chunks_per_head;
+    const int t = (int)(rest % T_len);
+    rest /= T_len;
+    const int h = (int)(rest % H);
+    const long long n = rest / H;
+    out[o] = in[((n * T_len + t) * H + h) * chunks_per_head + c];
+}
+
+// ---------------------------------------------------------------------------------------
+// Packed-projection cotangent from the attention pullback outputs.
+//   out[n, t, :] = [ R^T dq[n, 0..H) | R^T sum_group dk | sum_group dv ],  n = (b, p)
+// R is the rotary embedding of position t: (e, o) -> (e cos - o sin, e sin + o cos), pairs
+// (j, j + Dh/2) or, interleaved, (2j, 2j + 1); R^T: (ge cos + go sin, -ge sin + go cos).
+// One thread handles VEC pairs of one rotary head, or 2 VEC value elements.
+// ---------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void qkv_pullback_kernel(const T* __restrict__ dq, const T* __restrict__ dk,
+                                                           const T* __restrict__ dv, const float* __restrict__ cos_t,
+                                                           const float* __restrict__ sin_t, T* __restrict__ out,
+                                                           long long n_units, int T_len, int H, int Hkv, int Dh,
+                                                           int interleaved) {
+    const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (unit >= n_units) return;
+    const int half = Dh / 2;
+    const int upr = half / VEC;                  // units per head (rotary pair groups, or 2 VEC value elements)
+    const int per_token = (H + 2 * Hkv) * upr;
+    const long long row = unit / per_token;      // (n, t)
+    const int u = (int)(unit - row * per_token);
+    const int head = u / upr;                    // packed head index: q heads, then k heads, then v heads
+    const int j = (u - head * upr) * VEC;
+    const long long n = row / T_len;
+    const int t = (int)(row - n * T_len);
+    const int rep = H / Hkv;
+    T* o_row = out + row * (long long)(H + 2 * Hkv) * Dh + (long long)head * Dh;
+
+    // first / second storage offsets of this unit inside a head
+    const bool rotary = head < H + Hkv;
+    const int off0 = (rotary && !interleaved) ? j : 2 * j;
+    const int off1 = (rotary && !interleaved) ? half + j : 2 * j + VEC;
+
+    const T* src;
+    int first_head, count;
+    if (head < H) {
+        src = dq; first_head = head; count = 1;
+    } else if (head < H + Hkv) {
+        src = dk; first_head = (head - H) * rep; count = rep;
+    } else {
+        src = dv; first_head = (head - H - Hkv) * rep; count = rep;
+    }
+    float a0[VEC], a1[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) a0[i] = a1[i] = 0.0f;
+    for (int g = 0; g < count; ++g) {
+        const T* p = src + (((n * H + first_head + g) * T_len) + t) * (long long)Dh;
+        Pack<T, VEC> x0, x1;
+        x0.load(p + off0);
+        x1.load(p + off1);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            a0[i] += x0.v[i];
+            a1[i] += x1.v[i];
+        }
+    }
+    Pack<T, VEC> y0, y1;
+    if (!rotary) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            y0.v[i] = a0[i];
+            y1.v[i] = a1[i];
+        }
+    } else {
+        Pack<float, VEC> cs, sn;
+        cs.load(cos_t + (long long)t * half + j);
+        sn.load(sin_t + (long long)t * half + j);
+        float ge[VEC], go[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            if (interleaved) {  // a0|a1 holds pairs (2i, 2i+1) of the 2 VEC span
+                const int e = 2 * i, o = 2 * i + 1;
+                ge[i] = e < VEC ? a0[e % VEC] : a1[e % VEC];
+                go[i] = o < VEC ? a0[o % VEC] : a1[o % VEC];
+            } else {
+                ge[i] = a0[i];
+                go[i] = a1[i];
+            }
+        }
+        float re[VEC], ro[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            re[i] = ge[i] * cs.v[i] + go[i] * sn.v[i];
+            ro[i] = go[i] * cs.v[i] - ge[i] * sn.v[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            if (interleaved) {
+                const int e = 2 * i, o = 2 * i + 1;
+                if (e < VEC) y0.v[e % VEC] = re[i]; else y1.v[e % VEC] = re[i];
+                if (o < VEC) y0.v[o % VEC] = ro[i]; else y1.v[o % VEC] = ro[i];
+            } else {
+                y0.v[i] = re[i];
+                y1.v[i] = ro[i];
+            }
+        }
+    }
+    y0.store(o_row + off0);
+    y1.store(o_row + off1);
+}
+
+// ---------------------------------------------------------------------------------------
+// Depthwise causal convolution over T, transposed.
+//   forward  y[n, t, c] = sum_j w[c, j] x[n, t + j - (k-1), c]      (x = 0 before the sequence)
+//   pullback g_x[n, s, c] = sum_i w[c, k-1-i] g_y[n, s + i, c],  s + i < T
+// ---------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void causal_conv1d_pullback_kernel(const T* __restrict__ g_out,
+                                                                     const T* __restrict__ weight, T* __restrict__ g_in,
+                                                                     long long n_units, int T_len, int C, int ksize) {
+    const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (unit >= n_units) return;
+    const int per_row = C / VEC;
+    const long long row = unit / per_row;  // (n, s)
+    const int c0 = (int)(unit - row * per_row) * VEC;
+    const int s = (int)(row % T_len);
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+    const int steps = min(ksize, T_len - s);
+    for (int i = 0; i < steps; ++i) {
+        Pack<T, VEC> g;
+        g.load(g_out + (row + i) * C + c0);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+            acc[e] = fmaf(to_f32(weight[(long long)(c0 + e) * ksize + (ksize - 1 - i)]), g.v[e], acc[e]);
+    }
+    Pack<T, VEC> o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o.v[e] = acc[e];
+    o.store(g_in + row * C + c0);
+}
+
+inline unsigned blocks_for(long long units, int per_block) { return (unsigned)((units + per_block - 1) / per_block); }
+
+inline bool fits_grid(long long units, int per_block) {
+    return units > 0 && (units + per_block - 1) / per_block <= 0x7fffffffLL;
+}
+
+template <typename TB, typename TX>
+int launch_rmsnorm(const void* g_out, const void* x, const void* weight, const void* g_residual, void* g_sum,
+                   void* g_sum_branch, long long n_rows, int P, int T_len, int D, float eps, hipStream_t stream) {
+    const dim3 grid(blocks_for(n_rows, 4)), block(256);
+    if (D % 4 == 0)
+        hipLaunchKernelGGL((rmsnorm_pullback_kernel<TB, TX, 4>), grid, block, 0, stream, (const TB*)g_out, (const TX*)x,
+                           (const TB*)weight, (const float*)g_residual, (float*)g_sum, (TB*)g_sum_branch, n_rows, P,
+                           T_len, D, eps);
+    else
+        hipLaunchKernelGGL((rmsnorm_pullback_kernel<TB, TX, 1>), grid, block, 0, stream, (const TB*)g_out, (const TX*)x,
+                           (const TB*)weight, (const float*)g_residual, (float*)g_sum, (TB*)g_sum_branch, n_rows, P,
+                           T_len, D, eps);
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+template <typename TB>
+int launch_rmsnorm_x(int x_dtype, const void* g_out, const void* x, const void* weight, const void* g_residual,
+                     void* g_sum, void* g_sum_branch, long long n_rows, int P, int T_len, int D, float eps,
+                     hipStream_t stream) {
+    switch (x_dtype) {
+        case LBI_F32: return launch_rmsnorm<TB, float>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, stream);
+        case LBI_F16: return launch_rmsnorm<TB, _Float16>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, stream);
+        default: return launch_rmsnorm<TB, bf16_raw>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, stream);
+    }
+}
+
+template <typename T>
+int launch_gated(const void* g, const void* fc1, void* out, long long n_rows, int P, int T_len, int hidden,
+                 hipStream_t stream) {
+    if (hidden % 4 == 0) {
+        const long long units = n_rows * (hidden / 4);
+        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many elements");
+        hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, 4>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
+                           (const T*)g, (const T*)fc1, (T*)out, units, P, T_len, hidden);
+    } else {
+        const long long units = n_rows * hidden;
+        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many elements");
+        hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, 1>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
+                           (const T*)g, (const T*)fc1, (T*)out, units, P, T_len, hidden);
+    }
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+template <typename T>
+int launch_qkv(const void* dq, const void* dk, const void* dv, const float* cos_t, const float* sin_t, void* out,
+               long long n_rows, int T_len, int H, int Hkv, int Dh, int interleaved, hipStream_t stream) {
+    const int half = Dh / 2;
+    if (half % 4 == 0) {
+        const long long units = n_rows * (long long)(H + 2 * Hkv) * (half / 4);
+        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_qkv_pullback: too many elements");
+        hipLaunchKernelGGL((qkv_pullback_kernel<T, 4>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
+                           (const T*)dq, (const T*)dk, (const T*)dv, cos_t, sin_t, (T*)out, units, T_len, H, Hkv, Dh,
+                           interleaved);
+    } else {
+        const long long units = n_rows * (long long)(H + 2 * Hkv) * half;
+        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_qkv_pullback: too many elements");
+        hipLaunchKernelGGL((qkv_pullback_kernel<T, 1>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
+                           (const T*)dq, (const T*)dk, (const T*)dv, cos_t, sin_t, (T*)out, units, T_len, H, Hkv, Dh,
+                           interleaved);
+    }
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+template <typename T>
+int launch_conv(const void* g_out, const void* weight, void* g_in, long long n_rows, int T_len, int C, int ksize,
+                hipStream_t stream) {
+    if (C % 4 == 0) {
+        const long long units = n_rows * (C / 4);
+        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_causal_conv1d_pullback: too many elements");
+        hipLaunchKernelGGL((causal_conv1d_pullback_kernel<T, 4>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
+                           (const T*)g_out, (const T*)weight, (T*)g_in, units, T_len, C, ksize);
+    } else {
+        const long long units = n_rows * C;
+        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_causal_conv1d_pullback: too many elements");
+        hipLaunchKernelGGL((causal_conv1d_pullback_kernel<T, 1>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
+                           (const T*)g_out, (const T*)weight, (T*)g_in, units, T_len, C, ksize);
+    }
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+inline bool valid_dtype(int dtype) { return dtype == LBI_F32 || dtype == LBI_F16 || dtype == LBI_BF16; }
+inline bool positive_int(int64_t v) { return v > 0 && v <= 0x7fffffff; }
+
+}  // namespace region
+}  // namespace lbi
+
+using namespace lbi;
+
+extern "C" int lbi_rmsnorm_pullback(const void* g_out, const void* x, const void* weight, const void* g_residual,
+                                    void* g_sum, void* g_sum_branch, int64_t B, int64_t P, int64_t T, int64_t D,
+                                    float eps, int branch_dtype, int x_dtype, void* stream) {
+    clear_error();
+    if (!g_out || !x || !weight) return fail(LBI_ERR_INVALID, "lbi_rmsnorm_pullback: null input pointer");
+    if (!g_sum && !g_sum_branch) return fail(LBI_ERR_INVALID, "lbi_rmsnorm_pullback: no output requested");
+    if (!region::valid_dtype(branch_dtype) || !region::valid_dtype(x_dtype))
+        return fail(LBI_ERR_INVALID, "lbi_rmsnorm_pullback: bad dtype");
+    if (B < 0 || P < 0 || T < 0 || !region::positive_int(D) || P > 0x7fffffff || T > 0x7fffffff)
+        return fail(LBI_ERR_INVALID, "lbi_rmsnorm_pullback: bad size B=%lld P=%lld T=%lld D=%lld", (long long)B,
+                    (long long)P, (long long)T, (long long)D);
+    const long long n_rows = (long long)B * P * T;
+    if (n_rows == 0) return LBI_OK;
+    if (!region::fits_grid(n_rows, 4)) return fail(LBI_ERR_UNSUPPORTED, "lbi_rmsnorm_pullback: too many rows");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (branch_dtype) {
+        case LBI_F32: return region::launch_rmsnorm_x<float>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, s);
+        case LBI_F16: return region::launch_rmsnorm_x<_Float16>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, s);
+        default: return region::launch_rmsnorm_x<bf16_raw>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, s);
+    }
+}
+
+extern "C" int lbi_gated_mlp_pullback(const void* g_down_input, const void* fc1_output, void* g_fc1_output, int64_t B,
+                                      int64_t P, int64_t T, int64_t hidden, int dtype, void* stream) {
+    clear_error();
+    if (!g_down_input || !fc1_output || !g_fc1_output)
+        return fail(LBI_ERR_INVALID, "lbi_gated_mlp_pullback: null pointer");
+    if (!region::valid_dtype(dtype)) return fail(LBI_ERR_INVALID, "lbi_gated_mlp_pullback: bad dtype %d", dtype);
+    if (B < 0 || P < 0 || T < 0 || !region::positive_int(hidden) || P > 0x7fffffff || T > 0x7fffffff)
+        return fail(LBI_ERR_INVALID, "lbi_gated_mlp_pullback: bad size");
+    const long long n_rows = (long long)B * P * T;
+    if (n_rows == 0) return LBI_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case LBI_F32: return region::launch_gated<float>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, s);
+        case LBI_F16: return region::launch_gated<_Float16>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, s);
+        default: return region::launch_gated<bf16_raw>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, s);
+    }
+}
+
+extern "C" int lbi_attn_heads_split(const void* g_merged, void* g_heads, int64_t B, int64_t P, int64_t T, int64_t H,
+                                    int64_t Dh, int dtype, void* stream) {
+    clear_error();
+    if (!g_merged || !g_heads) return fail(LBI_ERR_INVALID, "lbi_attn_heads_split: null pointer");
+    if (!region::valid_dtype(dtype)) return fail(LBI_ERR_INVALID, "lbi_attn_heads_split: bad dtype %d", dtype);
+    if (B < 0 || P < 0 || !region::positive_int(T) || !region::positive_int(H) || !region::positive_int(Dh))
+        return fail(LBI_ERR_INVALID, "lbi_attn_heads_split: bad size");
+    const long long n = (long long)B * P;
+    if (n == 0) return LBI_OK;
+    const size_t head_bytes = (size_t)Dh * dtype_size(dtype);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool aligned = (reinterpret_cast<uintptr_t>(g_merged) | reinterpret_cast<uintptr_t>(g_heads)) % 16 == 0;
+    if (head_bytes % 16 == 0 && aligned) {
+        typedef unsigned int chunk16 __attribute__((ext_vector_type(4)));
+        const int cph = (int)(head_bytes / 16);
+        const long long chunks = n * T * H * cph;
+        if (!region::fits_grid(chunks, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_heads_split: too many elements");
+        hipLaunchKernelGGL((region::heads_split_kernel<chunk16>), dim3(region::blocks_for(chunks, 256)), dim3(256), 0, s,
+                           (const chunk16*)g_merged, (chunk16*)g_heads, chunks, (int)T, (int)H, cph);
+    } else if (dtype == LBI_F32) {
+        const long long chunks = n * T * H * Dh;
+        if (!region::fits_grid(chunks, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_heads_split: too many elements");
+        hipLaunchKernelGGL((region::heads_split_kernel<unsigned int>), dim3(region::blocks_for(chunks, 256)), dim3(256), 0,
+                           s, (const unsigned int*)g_merged, (unsigned int*)g_heads, chunks, (int)T, (int)H, (int)Dh);
+    } else {
+        const long long chunks = n * T * H * Dh;
+        if (!region::fits_grid(chunks, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_heads_split: too many elements");
+        hipLaunchKernelGGL((region::heads_split_kernel<unsigned short>), dim3(region::blocks_for(chunks, 256)), dim3(256),
+                           0, s, (const unsigned short*)g_merged, (unsigned short*)g_heads, chunks, (int)T, (int)H,
+                           (int)Dh);
+    }
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+extern "C" int lbi_attn_qkv_pullback(const void* dq, const void* dk, const void* dv, const float* rope_cos,
+                                     const float* rope_sin, void* g_qkv, int64_t B, int64_t P, int64_t T, int64_t H,
+                                     int64_t Hkv, int64_t Dh, int interleaved, int dtype, void* stream) {
+    clear_error();
+    if (!dq || !dk || !dv || !rope_cos || !rope_sin || !g_qkv)
+        return fail(LBI_ERR_INVALID, "lbi_attn_qkv_pullback: null pointer");
+    if (!region::valid_dtype(dtype)) return fail(LBI_ERR_INVALID, "lbi_attn_qkv_pullback: bad dtype %d", dtype);
+    if (B < 0 || P < 0 || !region::positive_int(T) || !region::positive_int(H) || !region::positive_int(Hkv) ||
+        !region::positive_int(Dh))
+        return fail(LBI_ERR_INVALID, "lbi_attn_qkv_pullback: bad size");
+    if (H % Hkv != 0) return fail(LBI_ERR_INVALID, "lbi_attn_qkv_pullback: H=%lld not a multiple of Hkv=%lld", (long long)H, (long long)Hkv);
+    if (Dh % 2 != 0) return fail(LBI_ERR_INVALID, "lbi_attn_qkv_pullback: rotary embedding needs an even head dim, got %lld", (long long)Dh);
+    const long long n_rows = (long long)B * P * T;
+    if (n_rows == 0) return LBI_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case LBI_F32: return region::launch_qkv<float>(dq, dk, dv, rope_cos, rope_sin, g_qkv, n_rows, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, s);
+        case LBI_F16: return region::launch_qkv<_Float16>(dq, dk, dv, rope_cos, rope_sin, g_qkv, n_rows, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, s);
+        default: return region::launch_qkv<bf16_raw>(dq, dk, dv, rope_cos, rope_sin, g_qkv, n_rows, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, s);
+    }
+}
+
+extern "C" int lbi_causal_conv1d_pullback(const void* g_out, const void* weight, void* g_in, int64_t N, int64_t T,
+                                          int64_t C, int64_t ksize, int dtype, void* stream) {
+    clear_error();
+    if (!g_out || !weight || !g_in) return fail(LBI_ERR_INVALID, "lbi_causal_conv1d_pullback: null pointer");
+    if (g_out == g_in) return fail(LBI_ERR_INVALID, "lbi_causal_conv1d_pullback: in-place call not supported");
+    if (!region::valid_dtype(dtype)) return fail(LBI_ERR_INVALID, "lbi_causal_conv1d_pullback: bad dtype %d", dtype);
+    if (N < 0 || !region::positive_int(T) || !region::positive_int(C) || ksize < 1 || ksize > 64)
+        return fail(LBI_ERR_INVALID, "lbi_causal_conv1d_pullback: bad size");
+    const long long n_rows = (long long)N * T;
+    if (n_rows == 0) return LBI_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case LBI_F32: return region::launch_conv<float>(g_out, weight, g_in, n_rows, (int)T, (int)C, (int)ksize, s);
+        case LBI_F16: return region::launch_conv<_Float16>(g_out, weight, g_in, n_rows, (int)T, (int)C, (int)ksize, s);
+        default: return region::launch_conv<bf16_raw>(g_out, weight, g_in, n_rows, (int)T, (int)C, (int)ksize, s);
+    }
+}

@@ -1,0 +1,234 @@
+"""Region-level input pullback of a Transformer layer range for P cotangent directions.
+
+Implements ``TransformerLowering.input_pullback_basis`` of the reference
+(backends/transformer.py:64-75; the CUDA class leaves it as a stub,
+backends/transformer_cuda.py:45-64) for the block the reference's backend executes
+(backends/transformer.py:118-246):
+
+    res1 = hidden (+ residual);  a = out_proj(attention(rope(split(conv1d(in_proj(norm(res1)))))))
+    res2 = a + res1;             m = fc2(up * silu(gate)),  [up | gate] = fc1(norm2(res2))
+    region_output = m + res2 of the last layer
+
+The cotangent basis [B, P, T, D] is pulled back through the layers in reverse.  Matrix
+products are library GEMMs on the [B*P*T, *] cotangent rows; everything between them runs in
+the kernels of liblbi_hip.so (RMSNorm, gated MLP, head split, rotary embedding + KV-group
+sum, causal convolution, and the attention pullback itself).  The residual-stream cotangent
+is kept in fp32, branch cotangents in the dtype of the weights.  Inputs are read from the
+forward cache the backend recorded; nothing is recomputed except the softmax statistics
+inside the attention kernel.  GPU only.
+"""
+from __future__ import annotations
+
+import math
+from typing import Any
+
+import torch
+
+from ... import _lib
+from . import attention_input_pullback_basis
+
+
+def _stream(t: torch.Tensor) -> int:
+    return _lib.current_stream_ptr(t.device)
+
+
+def _require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("region pullback tensors must be CUDA tensors (this build has no CPU execution path)")
+
+
+def rmsnorm_pullback(g_out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
+                     g_residual: torch.Tensor | None, *, want_branch: bool) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """``g_out [B,P,T,D]`` through RMSNorm at input ``x [B,T,D]``, plus ``g_residual`` (fp32).
+
+    Returns ``(sum fp32, sum in g_out.dtype or None)``.  ``g_residual`` is overwritten with the sum.
+    """
+    _require_cuda(g_out, x, weight)
+    bsz, basis, seqlen, dim = g_out.shape
+    if x.shape != (bsz, seqlen, dim) or weight.shape != (dim,):
+        raise ValueError("rmsnorm_pullback: x must be [B, T, D] and weight [D] matching g_out [B, P, T, D]")
+    g_out, x, weight = g_out.contiguous(), x.contiguous(), weight.to(g_out.dtype).contiguous()
+    if g_residual is None:
+        total = torch.empty(g_out.shape, device=g_out.device, dtype=torch.float32)
+        res_ptr = None
+    else:
+        if g_residual.dtype != torch.float32 or g_residual.shape != g_out.shape or not g_residual.is_contiguous():
+            raise ValueError("rmsnorm_pullback: g_residual must be a contiguous fp32 tensor shaped like g_out")
+        total = g_residual
+        res_ptr = g_residual.data_ptr()
+    branch = torch.empty_like(g_out) if want_branch else None
+    with torch.cuda.device(g_out.device):
+        status = _lib.load().lbi_rmsnorm_pullback(
+            g_out.data_ptr(), x.data_ptr(), weight.data_ptr(), res_ptr, total.data_ptr(),
+            branch.data_ptr() if branch is not None else None, bsz, basis, seqlen, dim, float(eps),
+            _lib.dtype_code(g_out.dtype), _lib.dtype_code(x.dtype), _stream(g_out))
+    _lib.check(status, "lbi_rmsnorm_pullback")
+    return total, branch
+
+
+def gated_mlp_pullback(g_down_input: torch.Tensor, fc1_output: torch.Tensor) -> torch.Tensor:
+    """``g_down_input [B,P,T,Hd]``, ``fc1_output [B,T,2Hd]`` -> cotangent of fc1_output ``[B,P,T,2Hd]``."""
+    _require_cuda(g_down_input, fc1_output)
+    bsz, basis, seqlen, hidden = g_down_input.shape
+    if fc1_output.shape != (bsz, seqlen, 2 * hidden) or fc1_output.dtype != g_down_input.dtype:
+        raise ValueError("gated_mlp_pullback: fc1_output must be [B, T, 2*hidden] in the dtype of g_down_input")
+    g_down_input, fc1_output = g_down_input.contiguous(), fc1_output.contiguous()
+    out = torch.empty((bsz, basis, seqlen, 2 * hidden), device=g_down_input.device, dtype=g_down_input.dtype)
+    with torch.cuda.device(out.device):
+        status = _lib.load().lbi_gated_mlp_pullback(
+            g_down_input.data_ptr(), fc1_output.data_ptr(), out.data_ptr(), bsz, basis, seqlen, hidden,
+            _lib.dtype_code(out.dtype), _stream(out))
+    _lib.check(status, "lbi_gated_mlp_pullback")
+    return out
+
+
+def attn_heads_split(g_merged: torch.Tensor, n_heads: int, head_dim: int) -> torch.Tensor:
+    """``[B,P,T,H*Dh]`` -> ``[B,P,H,T,Dh]``."""
+    _require_cuda(g_merged)
+    bsz, basis, seqlen, width = g_merged.shape
+    if width != n_heads * head_dim:
+        raise ValueError("attn_heads_split: last dimension must be n_heads * head_dim")
+    g_merged = g_merged.contiguous()
+    out = torch.empty((bsz, basis, n_heads, seqlen, head_dim), device=g_merged.device, dtype=g_merged.dtype)
+    with torch.cuda.device(out.device):
+        status = _lib.load().lbi_attn_heads_split(g_merged.data_ptr(), out.data_ptr(), bsz, basis, seqlen, n_heads,
+                                                  head_dim, _lib.dtype_code(out.dtype), _stream(out))
+    _lib.check(status, "lbi_attn_heads_split")
+    return out
+
+
+_ROPE_TABLES: dict[tuple, tuple[torch.Tensor, torch.Tensor]] = {}
+
+
+def rope_tables(seq_len: int, head_dim: int, base: float, device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos, sin ``[T, Dh/2]`` fp32 of the rotary angles, built as the reference's apply_rope does
+    (backbones/transformer/rope.py:14-20) and cached per (T, Dh, base, device)."""
+    key = (seq_len, head_dim, float(base), str(device))
+    hit = _ROPE_TABLES.get(key)
+    if hit is None:
+        half = head_dim // 2
+        positions = torch.arange(seq_len, device=device, dtype=torch.float32)
+        freq_seq = torch.arange(half, device=device, dtype=torch.float32)
+        freqs = torch.outer(positions, base ** (-2.0 * freq_seq / float(head_dim)))
+        hit = (freqs.cos().contiguous(), freqs.sin().contiguous())
+        if len(_ROPE_TABLES) > 32:
+            _ROPE_TABLES.clear()
+        _ROPE_TABLES[key] = hit
+    return hit
+
+
+def attn_qkv_pullback(dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor, *, n_kv_heads: int, rope_base: float,
+                      rope_interleaved: bool) -> torch.Tensor:
+    """``dq, dk, dv [B,P,H,T,Dh]`` -> cotangent of the packed projection ``[B,P,T,(H+2Hkv)*Dh]``."""
+    _require_cuda(dq, dk, dv)
+    bsz, basis, heads, seqlen, head_dim = dq.shape
+    if dk.shape != dq.shape or dv.shape != dq.shape or dk.dtype != dq.dtype or dv.dtype != dq.dtype:
+        raise ValueError("attn_qkv_pullback: dq, dk, dv must share shape [B, P, H, T, Dh] and dtype")
+    if heads % n_kv_heads:
+        raise ValueError("n_heads must be divisible by n_kv_heads")
+    if head_dim % 2:
+        raise ValueError("RoPE requires an even head dimension.")
+    dq, dk, dv = dq.contiguous(), dk.contiguous(), dv.contiguous()
+    cos, sin = rope_tables(seqlen, head_dim, rope_base, dq.device)
+    out = torch.empty((bsz, basis, seqlen, (heads + 2 * n_kv_heads) * head_dim), device=dq.device, dtype=dq.dtype)
+    with torch.cuda.device(out.device):
+        status = _lib.load().lbi_attn_qkv_pullback(
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), cos.data_ptr(), sin.data_ptr(), out.data_ptr(), bsz, basis,
+            seqlen, heads, n_kv_heads, head_dim, int(bool(rope_interleaved)), _lib.dtype_code(out.dtype), _stream(out))
+    _lib.check(status, "lbi_attn_qkv_pullback")
+    return out
+
+
+def causal_conv1d_pullback(g_out: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``g_out [B,P,T,C]`` through the depthwise causal convolution with ``weight [C,1,k]``."""
+    _require_cuda(g_out, weight)
+    bsz, basis, seqlen, channels = g_out.shape
+    if weight.dim() != 3 or weight.shape[0] != channels or weight.shape[1] != 1:
+        raise ValueError("causal_conv1d_pullback: weight must be [C, 1, k] (depthwise)")
+    g_out = g_out.contiguous()
+    weight = weight.to(g_out.dtype).contiguous()
+    out = torch.empty_like(g_out)
+    with torch.cuda.device(out.device):
+        status = _lib.load().lbi_causal_conv1d_pullback(g_out.data_ptr(), weight.data_ptr(), out.data_ptr(),
+                                                        bsz * basis, seqlen, channels, weight.shape[-1],
+                                                        _lib.dtype_code(out.dtype), _stream(out))
+    _lib.check(status, "lbi_causal_conv1d_pullback")
+    return out
+
+
+def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor | None, g_residual: torch.Tensor,
+                          kernel_mode: str) -> torch.Tensor:
+    """One block, backwards.  ``g_residual`` (fp32, [B,P,T,D]) is the cotangent of the block's
+    residual output and is updated in place; ``g_hidden`` is the cotangent of its hidden output
+    in the weight dtype (``None``: equal to ``g_residual``).  Returns the cotangent of
+    ``hidden (+ residual)`` at the block input, fp32."""
+    attn, mlp = block.attn, block.mlp
+    wdtype = mlp.fc2.weight.dtype
+    a_cache, m_cache = layer_cache.attention, layer_cache.mlp
+    if g_hidden is None:
+        g_hidden = g_residual.to(wdtype)
+
+    # gated MLP: hidden_out = fc2(up * silu(gate)), [up | gate] = fc1(norm2(res2))
+    g_down_input = torch.matmul(g_hidden, mlp.fc2.weight)
+    g_fc1 = gated_mlp_pullback(g_down_input, m_cache.fc1_output)
+    del g_down_input
+    g_norm2 = torch.matmul(g_fc1, mlp.fc1.weight)
+    del g_fc1
+    # res2 feeds norm2 and the residual output
+    g_res2, g_attn_out = rmsnorm_pullback(g_norm2, m_cache.norm_input, block.norm2.weight, block.norm2.eps,
+                                          g_residual, want_branch=True)
+    del g_norm2
+
+    # attention: res2 = out_proj(heads) + res1
+    g_merged = torch.matmul(g_attn_out, attn.out_proj.weight)
+    del g_attn_out
+    g_heads = attn_heads_split(g_merged, attn.n_heads, attn.head_dim)
+    del g_merged
+    scale = attn.softmax_scale if attn.softmax_scale is not None else 1.0 / math.sqrt(attn.head_dim)
+    dq, dk, dv = attention_input_pullback_basis(a_cache.q_rope, a_cache.k_expanded, a_cache.v_expanded, g_heads,
+                                                softmax_scale=float(scale), causal=True, kernel_mode=kernel_mode)
+    del g_heads
+    g_qkv = attn_qkv_pullback(dq, dk, dv, n_kv_heads=attn.n_kv_heads, rope_base=attn.rope_base,
+                              rope_interleaved=attn.rope_interleaved)
+    del dq, dk, dv
+    if attn.d_conv > 0:
+        g_qkv = causal_conv1d_pullback(g_qkv, attn.conv1d.weight)
+    g_norm1 = torch.matmul(g_qkv, attn.in_proj.weight)
+    del g_qkv
+    g_res1, _ = rmsnorm_pullback(g_norm1, a_cache.norm_input, block.norm.weight, block.norm.eps, g_res2,
+                                 want_branch=False)
+    return g_res1
+
+
+def region_input_pullback_basis(backend: Any, cache: Any, output_cotangent_basis: torch.Tensor, *,
+                                kernel_mode: str = "hip") -> torch.Tensor:
+    """``output_cotangent_basis [B, P, T, D]`` -> region-input cotangents ``[B, P, T, D]``.
+
+    ``backend.backbone.blocks`` and ``cache.layer_caches`` use the attribute names of the
+    reference's ``TransformerRegionBackend`` / ``TransformerRegionCache``.
+    """
+    if output_cotangent_basis.dim() != 4:
+        raise ValueError("output_cotangent_basis must have shape [B, P, T, D]")
+    if not output_cotangent_basis.is_cuda:
+        raise RuntimeError("output_cotangent_basis must be a CUDA tensor (this build has no CPU execution path)")
+    start, end = cache.layer_range
+    if len(cache.layer_caches) != end - start:
+        raise ValueError("cache.layer_caches does not match cache.layer_range")
+    if end == start:
+        return output_cotangent_basis.clone()
+    device = cache.region_input.device
+    # region_output = hidden + residual of the last block: both receive the cotangent
+    g = output_cotangent_basis.to(device=device, dtype=torch.float32, copy=True).contiguous()
+    for offset in range(end - start - 1, -1, -1):
+        layer_cache = cache.layer_caches[offset]
+        block = backend.backbone.blocks[layer_cache.layer_index]
+        g = _layer_input_pullback(block, layer_cache, None, g, kernel_mode)
+        # hidden and residual at the block input enter only through their sum
+    return g.to(device=output_cotangent_basis.device, dtype=output_cotangent_basis.dtype)
+
+
+__all__ = [
+    "attn_heads_split", "attn_qkv_pullback", "causal_conv1d_pullback", "gated_mlp_pullback", "rmsnorm_pullback",
+    "region_input_pullback_basis", "rope_tables",
+]

@@ -1,0 +1,219 @@
+"""Region-level input pullback on the GPU (through the C ABI) against autograd of the
+CPU restatement of the reference's Transformer region."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import transformer_region as oreg
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+
+
+def _tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 2e-2
+
+
+def _max_rel(a, b):
+    return float((a.double() - b.double()).abs().max() / b.double().abs().max().clamp_min(1e-30))
+
+
+def _vjp(fn, inputs, cotangent):
+    inputs = [t.detach().double().requires_grad_(True) for t in inputs]
+    out = fn(*inputs)
+    return torch.autograd.grad(out, inputs, grad_outputs=cotangent.double())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim", [32, 30, 768])
+def test_rmsnorm_pullback(dtype, dim, device):
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(dim)
+    b, p, t = 2, 3, 5
+    g = torch.randn(b, p, t, dim).to(dtype)
+    x = torch.randn(b, t, dim)  # fp32 residual stream
+    w = (1 + 0.1 * torch.randn(dim)).to(dtype)
+    res = torch.randn(b, p, t, dim)
+    total, branch = region.rmsnorm_pullback(g.to(device), x.to(device), w.to(device), 1e-5, res.clone().to(device),
+                                            want_branch=True)
+    xr = x.to(dtype)  # the norm runs on the input rounded to the weight dtype
+
+    def fwd(xx):
+        return xx * torch.rsqrt(xx.pow(2).mean(-1, keepdim=True) + 1e-5) * w.double()
+
+    want = torch.stack([_vjp(fwd, [xr], g[:, i])[0] for i in range(p)], dim=1) + res.double()
+    assert total.dtype == torch.float32 and branch.dtype == dtype
+    assert _max_rel(total.cpu(), want) <= 2e-5  # fp32 arithmetic on the given (rounded) inputs
+    assert _max_rel(branch.cpu(), want) <= _tol(dtype)
+    # no residual, fp32 output only
+    only, none = region.rmsnorm_pullback(g.to(device), x.to(device), w.to(device), 1e-5, None, want_branch=False)
+    assert none is None and _max_rel(only.cpu(), want - res.double()) <= 2e-5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [24, 27, 3072])
+def test_gated_mlp_pullback(dtype, hidden, device):
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(hidden)
+    b, p, t = 2, 2, 3
+    g = torch.randn(b, p, t, hidden).to(dtype)
+    fc1 = (2 * torch.randn(b, t, 2 * hidden)).to(dtype)
+    got = region.gated_mlp_pullback(g.to(device), fc1.to(device)).cpu()
+
+    def fwd(f):
+        return f[..., :hidden] * F.silu(f[..., hidden:])
+
+    want = torch.stack([_vjp(fwd, [fc1], g[:, i])[0] for i in range(p)], dim=1)
+    assert got.dtype == dtype and got.shape == (b, p, t, 2 * hidden)
+    assert _max_rel(got, want) <= _tol(dtype)
+    assert torch.allclose(got.double(), want, atol=_tol(dtype) * 4, rtol=_tol(dtype) * 4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,head_dim", [(3, 4), (2, 64), (5, 6)])
+def test_heads_split(dtype, heads, head_dim, device):
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    x = torch.randn(2, 3, 7, heads * head_dim).to(dtype)
+    got = region.attn_heads_split(x.to(device), heads, head_dim).cpu()
+    assert torch.equal(got, x.view(2, 3, 7, heads, head_dim).permute(0, 1, 3, 2, 4).contiguous())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,interleaved",
+                         [(4, 4, 8, False), (4, 2, 8, True), (6, 2, 6, False), (3, 1, 2, True), (12, 4, 64, False),
+                          (2, 1, 64, True)])
+def test_qkv_pullback(dtype, heads, kv_heads, head_dim, interleaved, device):
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(heads * 100 + head_dim)
+    b, p, t = 2, 3, 9
+    dq, dk, dv = (torch.randn(b, p, heads, t, head_dim).to(dtype) for _ in range(3))
+    got = region.attn_qkv_pullback(dq.to(device), dk.to(device), dv.to(device), n_kv_heads=kv_heads, rope_base=100.0,
+                                   rope_interleaved=interleaved).cpu()
+    rep = heads // kv_heads
+
+    def fwd(qkv):  # [b, t, (H + 2 Hkv) Dh] -> concatenated (q_rope, k_expanded, v_expanded)
+        q, k, v = qkv.split((heads * head_dim, kv_heads * head_dim, kv_heads * head_dim), dim=-1)
+        q = q.view(b, t, heads, head_dim).transpose(1, 2)
+        k = k.view(b, t, kv_heads, head_dim).transpose(1, 2)
+        v = v.view(b, t, kv_heads, head_dim).transpose(1, 2)
+        # float64 rotation from the same fp32 tables as the kernel
+        cos, sin = (c.double() for c in oreg.rope_tables(t, head_dim, 100.0))
+
+        def rot(x):
+            if interleaved:
+                a, c = x[..., 0::2], x[..., 1::2]
+                return torch.stack((a * cos - c * sin, a * sin + c * cos), dim=-1).flatten(-2)
+            a, c = x[..., : head_dim // 2], x[..., head_dim // 2:]
+            return torch.cat((a * cos - c * sin, a * sin + c * cos), dim=-1)
+
+        return torch.cat((rot(q), rot(k).repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)), dim=1)
+
+    qkv0 = torch.zeros(b, t, (heads + 2 * kv_heads) * head_dim)
+    want = torch.stack([_vjp(fwd, [qkv0], torch.cat((dq[:, i], dk[:, i], dv[:, i]), dim=1))[0] for i in range(p)], dim=1)
+    assert got.dtype == dtype and got.shape == want.shape
+    assert _max_rel(got, want) <= (1e-6 if dtype == torch.float32 else _tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("channels,ksize,seqlen", [(8, 4, 10), (6, 3, 2), (5, 1, 4), (2304, 4, 7)])
+def test_causal_conv1d_pullback(dtype, channels, ksize, seqlen, device):
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(channels + ksize)
+    b, p = 2, 2
+    g = torch.randn(b, p, seqlen, channels).to(dtype)
+    w = torch.randn(channels, 1, ksize).to(dtype)
+    got = region.causal_conv1d_pullback(g.to(device), w.to(device)).cpu()
+
+    def fwd(x):  # [b, T, C]
+        return F.conv1d(x.transpose(1, 2), w.double(), padding=ksize - 1, groups=channels)[..., :seqlen].transpose(1, 2)
+
+    want = torch.stack([_vjp(fwd, [torch.zeros(b, seqlen, channels)], g[:, i])[0] for i in range(p)], dim=1)
+    assert _max_rel(got, want) <= (1e-6 if dtype == torch.float32 else _tol(dtype))
+
+
+REGION_CASES = [
+    # dim, heads, kv, head_dim, hidden, layers, d_conv, interleaved, B, P, T
+    (32, 4, 2, 8, 48, 2, 4, False, 2, 3, 12),
+    (24, 3, 3, 8, 40, 1, 0, True, 1, 2, 9),
+    (16, 2, 1, 6, 20, 3, 2, False, 2, 2, 5),
+]
+
+
+@pytest.mark.parametrize("case", REGION_CASES)
+def test_region_pullback_fp32_matches_autograd(case, device):
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+
+    dim, heads, kv, hd, hidden, layers, d_conv, inter, b, p, t = case
+    backend = oreg.make_backend(dim=dim, n_heads=heads, n_kv_heads=kv, head_dim=hd, hidden=hidden, layers=layers,
+                                d_conv=d_conv, rope_interleaved=inter, rope_base=1000.0, seed=dim)
+    torch.manual_seed(t)
+    x = torch.randn(b, t, dim)
+    basis = torch.randn(b, p, t, dim)
+    _, cpu_cache = backend.forward_region(region_input=x, region_index=0)
+    want = oreg.input_pullback_basis_autograd(backend, cpu_cache, basis)
+
+    gpu_backend = backend.to(device)
+    with torch.no_grad():
+        _, cache = gpu_backend.forward_region(region_input=x.to(device), region_index=0)
+    got = HipTransformerLowering().input_pullback_basis(backend=gpu_backend, cache=cache,
+                                                        output_cotangent_basis=basis.to(device))
+    assert got.shape == basis.shape and got.dtype == basis.dtype and got.is_cuda
+    assert _max_rel(got.cpu(), want) <= 2e-5, _max_rel(got.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("residual_in_fp32", [True, False])
+def test_region_pullback_16bit_matches_fp32_path(dtype, residual_in_fp32, device):
+    """16-bit weights and activations (MFMA attention path: Dh=64, T=128) against fp32 autograd
+    of the same (rounded) weights."""
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+
+    dim, heads, kv, hd, hidden, layers, b, p, t = 128, 2, 1, 64, 256, 2, 2, 5, 128
+    backend = oreg.make_backend(dim=dim, n_heads=heads, n_kv_heads=kv, head_dim=hd, hidden=hidden, layers=layers,
+                                d_conv=4, residual_in_fp32=residual_in_fp32, dtype=dtype, seed=11)
+    torch.manual_seed(12)
+    x = torch.randn(b, t, dim).to(dtype)
+    basis = torch.randn(b, p, t, dim)
+    import copy
+
+    ref_backend = copy.deepcopy(backend).float()  # same rounded weights, fp32 arithmetic
+    _, ref_cache = ref_backend.forward_region(region_input=x.float(), region_index=0)
+    want = oreg.input_pullback_basis_autograd(ref_backend, ref_cache, basis)
+
+    gpu_backend = backend.to(device)
+    with torch.no_grad():
+        _, cache = gpu_backend.forward_region(region_input=x.to(device), region_index=0)
+    got = HipTransformerLowering().input_pullback_basis(backend=gpu_backend, cache=cache,
+                                                        output_cotangent_basis=basis.to(device))
+    assert got.dtype == basis.dtype
+    assert _max_rel(got.cpu(), want) <= 2e-2, _max_rel(got.cpu(), want)
+
+
+def test_region_pullback_contract(device):
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+
+    backend = oreg.make_backend(dim=16, n_heads=2, head_dim=8, hidden=16, layers=1, seed=1).to(device)
+    x = torch.randn(1, 4, 16, device=device)
+    with torch.no_grad():
+        _, cache = backend.forward_region(region_input=x, region_index=0)
+    low = HipTransformerLowering()
+    with pytest.raises(ValueError, match=r"\[B, P, T, D\]"):
+        low.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=torch.zeros(1, 4, 16, device=device))
+    # linear in the cotangent, and direction p depends on basis[:, p] only
+    basis = torch.randn(1, 3, 4, 16, device=device)
+    out = low.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=basis)
+    one = low.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=basis[:, 1:2])
+    assert torch.allclose(out[:, 1:2], one, atol=1e-6)
+    twice = low.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=2 * basis)
+    assert torch.allclose(twice, 2 * out, atol=1e-5)
+    # a zero-layer range is the identity
+    cache.layer_range, cache.layer_caches = (0, 0), []
+    assert torch.equal(low.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=basis), basis)
