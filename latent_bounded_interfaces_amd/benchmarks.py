@@ -1,4 +1,4 @@
-"""Timing harness for the attention input-pullback on one GPU.
+"""Timing harness for the attention input-pullback and the region input pullback on one GPU.
 
 Counterpart of reference benchmarks/time_attention_pullback.py: warm-up, then the
 median and best of ``iters`` device-timed calls (HIP events on the launch stream,
@@ -120,6 +120,91 @@ def attention_section(steps: int = 5) -> dict:
     return out
 
 
+# ---------------------------------------------------------------------------------------
+# Region-level input pullback (a range of Transformer layers, P cotangent directions)
+# ---------------------------------------------------------------------------------------
+def synthetic_region(*, dim, n_heads, n_kv_heads, head_dim, hidden, layers, d_conv, batch, seq_len, dtype, device,
+                     residual_in_fp32=True, seed=0):
+    """Random weights and a random forward cache with the attribute names of the reference's
+    ``TransformerRegionBackend`` / ``TransformerRegionCache`` (only the fields the pullback reads).
+    Values are synthetic (N(0,1) activations, N(0,1/fan_in) weights); shapes and dtypes are the real ones."""
+    from types import SimpleNamespace as NS
+
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+
+    def rand(*shape, std=1.0, dt=dtype):
+        return (torch.randn(*shape, generator=gen) * std).to(dt).to(device)
+
+    res_dtype = torch.float32 if residual_in_fp32 else dtype
+    qkv_dim = (n_heads + 2 * n_kv_heads) * head_dim
+    blocks, caches = [], []
+    for layer in range(layers):
+        attn = NS(n_heads=n_heads, n_kv_heads=n_kv_heads, head_dim=head_dim, rope_base=10000.0, rope_interleaved=False,
+                  softmax_scale=None, d_conv=d_conv,
+                  in_proj=NS(weight=rand(qkv_dim, dim, std=dim ** -0.5)),
+                  out_proj=NS(weight=rand(dim, n_heads * head_dim, std=(n_heads * head_dim) ** -0.5)))
+        if d_conv > 0:
+            attn.conv1d = NS(weight=rand(qkv_dim, 1, d_conv, std=d_conv ** -0.5))
+        mlp = NS(fc1=NS(weight=rand(2 * hidden, dim, std=dim ** -0.5)), fc2=NS(weight=rand(dim, hidden, std=hidden ** -0.5)))
+        blocks.append(NS(attn=attn, mlp=mlp, norm=NS(weight=rand(dim) * 0.1 + 1, eps=1e-5),
+                         norm2=NS(weight=rand(dim) * 0.1 + 1, eps=1e-5), residual_in_fp32=residual_in_fp32))
+        a_cache = NS(norm_input=rand(batch, seq_len, dim, dt=res_dtype if layer else dtype),
+                     q_rope=rand(batch, n_heads, seq_len, head_dim), k_expanded=rand(batch, n_heads, seq_len, head_dim),
+                     v_expanded=rand(batch, n_heads, seq_len, head_dim))
+        m_cache = NS(norm_input=rand(batch, seq_len, dim, dt=res_dtype), fc1_output=rand(batch, seq_len, 2 * hidden))
+        caches.append(NS(layer_index=layer, attention=a_cache, mlp=m_cache))
+    backend = NS(backbone=NS(blocks=blocks))
+    cache = NS(region_index=0, layer_range=(0, layers), layer_caches=caches,
+               region_input=rand(batch, seq_len, dim))
+    return backend, cache
+
+
+def region_flops(*, dim, n_heads, n_kv_heads, head_dim, hidden, layers, batch, seq_len, basis) -> dict:
+    """Algorithmic flops of the region input pullback: the four transposed projections per
+    layer on B*P*T cotangent rows, plus the attention pullback."""
+    rows = batch * basis * seq_len
+    qkv_dim = (n_heads + 2 * n_kv_heads) * head_dim
+    gemm = 2.0 * rows * (dim * hidden + 2 * hidden * dim + dim * n_heads * head_dim + qkv_dim * dim) * layers
+    attn = algorithmic_flops(batch, n_heads, seq_len, head_dim, basis, True) * layers
+    return {"gemm": gemm, "attention": attn, "total": gemm + attn}
+
+
+def measure_region(*, dim=768, n_heads=12, n_kv_heads=12, head_dim=64, hidden=3072, layers=2, d_conv=4, batch=8,
+                   seq_len=1024, basis=64, dtype=torch.bfloat16, warmup=2, iters=5, device="cuda") -> dict:
+    from .backends import HipTransformerLowering
+
+    backend, cache = synthetic_region(dim=dim, n_heads=n_heads, n_kv_heads=n_kv_heads, head_dim=head_dim, hidden=hidden,
+                                      layers=layers, d_conv=d_conv, batch=batch, seq_len=seq_len, dtype=dtype,
+                                      device=device)
+    gen = torch.Generator(device="cpu").manual_seed(1)
+    cot = torch.randn(batch, basis, seq_len, dim, generator=gen).to(device)
+    lowering = HipTransformerLowering()
+
+    def call():
+        return lowering.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=cot)
+
+    median_ms, best_ms, mean_ms, peak = time_call(call, warmup=warmup, iters=iters)
+    first = call().clone()
+    stable = bool(torch.equal(first, call()))
+    flops = region_flops(dim=dim, n_heads=n_heads, n_kv_heads=n_kv_heads, head_dim=head_dim, hidden=hidden, layers=layers,
+                         batch=batch, seq_len=seq_len, basis=basis)
+    tflops = flops["total"] / (mean_ms * 1e-3) / 1e12
+    return {
+        "workload": f"region input pullback: {layers} layers, d_model {dim}, {n_heads} heads x {head_dim}, "
+                    f"hidden {hidden}, conv {d_conv}, B={batch} T={seq_len} P={basis}, {str(dtype).replace('torch.', '')}",
+        "median_ms": median_ms, "best_ms": best_ms, "mean_ms": mean_ms, "peak_memory_bytes": peak,
+        "algorithmic_flops": flops, "tflops": tflops, "bit_stable_rerun": stable,
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_MFMA_16BIT_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_MFMA_16BIT_TFLOPS},
+    }
+
+
+def region_section(steps: int = 5) -> dict:
+    """One region of the end-to-end configuration (2 of 12 layers, d_model 768, 12 heads, interface width 64
+    = 64 cotangent directions, batch 8, sequence 1024, bf16)."""
+    return {"region_input_pullback_bf16_L2_D768_B8_T1024_P64": measure_region(iters=steps)}
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
     ap.add_argument("--shapes", nargs="*", default=["1,8,128,64,4"], help="B,H,T,Dh,P tuples")
@@ -129,7 +214,14 @@ def main(argv=None) -> int:
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--csv", default=None)
     ap.add_argument("--json", default=None)
+    ap.add_argument("--region", action="store_true",
+                    help="time the region-level input pullback at the end-to-end configuration instead")
+    ap.add_argument("--basis", type=int, default=64, help="cotangent directions of the --region run")
     args = ap.parse_args(argv)
+    if args.region:
+        print(json.dumps(measure_region(basis=args.basis, dtype=getattr(torch, args.dtype), warmup=args.warmup,
+                                        iters=args.iters)), flush=True)
+        return 0
     rows = []
     for spec in args.shapes:
         B, H, T, Dh, P = (int(x) for x in spec.split(","))

@@ -54,6 +54,38 @@ template <> __device__ __forceinline__ void Pack<bf16_raw, 4>::store(bf16_raw* p
         u16x4{f32_to_bf16_bits(v[0]), f32_to_bf16_bits(v[1]), f32_to_bf16_bits(v[2]), f32_to_bf16_bits(v[3])};
 }
 
+// Eight 16-bit elements: one 16-byte access.
+template <> struct Pack<_Float16, 8> {
+    float v[8];
+    __device__ __forceinline__ void load(const _Float16* p) {
+        const f16x8 h = *reinterpret_cast<const f16x8*>(p);
+        v[0] = (float)h[0]; v[1] = (float)h[1]; v[2] = (float)h[2]; v[3] = (float)h[3];
+        v[4] = (float)h[4]; v[5] = (float)h[5]; v[6] = (float)h[6]; v[7] = (float)h[7];
+    }
+    __device__ __forceinline__ void store(_Float16* p) const {
+        *reinterpret_cast<f16x8*>(p) = f16x8{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3],
+                                             (_Float16)v[4], (_Float16)v[5], (_Float16)v[6], (_Float16)v[7]};
+    }
+};
+template <> struct Pack<bf16_raw, 8> {
+    float v[8];
+    __device__ __forceinline__ void load(const bf16_raw* p) {
+        const f32x4 w = *reinterpret_cast<const f32x4*>(p);  // four words, two elements each
+        v[0] = __uint_as_float(__float_as_uint(w[0]) << 16); v[1] = __uint_as_float(__float_as_uint(w[0]) & 0xffff0000u);
+        v[2] = __uint_as_float(__float_as_uint(w[1]) << 16); v[3] = __uint_as_float(__float_as_uint(w[1]) & 0xffff0000u);
+        v[4] = __uint_as_float(__float_as_uint(w[2]) << 16); v[5] = __uint_as_float(__float_as_uint(w[2]) & 0xffff0000u);
+        v[6] = __uint_as_float(__float_as_uint(w[3]) << 16); v[7] = __uint_as_float(__float_as_uint(w[3]) & 0xffff0000u);
+    }
+    __device__ __forceinline__ void store(bf16_raw* p) const {
+        *reinterpret_cast<u16x8*>(p) =
+            u16x8{f32_to_bf16_bits(v[0]), f32_to_bf16_bits(v[1]), f32_to_bf16_bits(v[2]), f32_to_bf16_bits(v[3]),
+                  f32_to_bf16_bits(v[4]), f32_to_bf16_bits(v[5]), f32_to_bf16_bits(v[6]), f32_to_bf16_bits(v[7])};
+    }
+};
+
+// Elements of T in a 16-byte access.
+template <typename T> constexpr int wide() { return 16 / (int)sizeof(T); }
+
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
@@ -274,31 +306,60 @@ __global__ __launch_bounds__(256) void qkv_pullback_kernel(const T* __restrict__
 //   forward  y[n, t, c] = sum_j w[c, j] x[n, t + j - (k-1), c]      (x = 0 before the sequence)
 //   pullback g_x[n, s, c] = sum_i w[c, k-1-i] g_y[n, s + i, c],  s + i < T
 // ---------------------------------------------------------------------------------------
-template <typename T, int VEC>
+// One thread: VEC channels x RUN consecutive positions, KMAX >= ksize taps held in registers
+// (taps past ksize are zero), input rows read once per RUN outputs.
+template <typename T, int VEC, int KMAX, int RUN>
 __global__ __launch_bounds__(256) void causal_conv1d_pullback_kernel(const T* __restrict__ g_out,
                                                                      const T* __restrict__ weight, T* __restrict__ g_in,
                                                                      long long n_units, int T_len, int C, int ksize) {
     const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
     if (unit >= n_units) return;
     const int per_row = C / VEC;
-    const long long row = unit / per_row;  // (n, s)
-    const int c0 = (int)(unit - row * per_row) * VEC;
-    const int s = (int)(row % T_len);
-    float acc[VEC];
+    const int n_runs = (T_len + RUN - 1) / RUN;
+    const int c0 = (int)(unit % per_row) * VEC;
+    const long long rest = unit / per_row;
+    const int s0 = (int)(rest % n_runs) * RUN;
+    const long long n = rest / n_runs;
+
+    float tap[KMAX][VEC];  // tap[i][e] multiplies g_out at offset +i
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
-    const int steps = min(ksize, T_len - s);
-    for (int i = 0; i < steps; ++i) {
-        Pack<T, VEC> g;
-        g.load(g_out + (row + i) * C + c0);
+    for (int i = 0; i < KMAX; ++i)
 #pragma unroll
         for (int e = 0; e < VEC; ++e)
-            acc[e] = fmaf(to_f32(weight[(long long)(c0 + e) * ksize + (ksize - 1 - i)]), g.v[e], acc[e]);
-    }
-    Pack<T, VEC> o;
+            tap[i][e] = i < ksize ? to_f32(weight[(long long)(c0 + e) * ksize + (ksize - 1 - i)]) : 0.0f;
+    float acc[RUN][VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) o.v[e] = acc[e];
-    o.store(g_in + row * C + c0);
+    for (int r = 0; r < RUN; ++r)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[r][e] = 0.0f;
+    const long long base = (n * T_len + s0) * C + c0;
+#pragma unroll
+    for (int j = 0; j < RUN + KMAX - 1; ++j) {
+        Pack<T, VEC> g;
+        if (s0 + j < T_len && j < RUN + ksize - 1) {
+            g.load(g_out + base + (long long)j * C);
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) g.v[e] = 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < RUN; ++r) {
+            const int i = j - r;
+            if (i >= 0 && i < KMAX) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[r][e] = fmaf(tap[i][e], g.v[e], acc[r][e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RUN; ++r) {
+        if (s0 + r < T_len) {
+            Pack<T, VEC> o;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o.v[e] = acc[r][e];
+            o.store(g_in + base + (long long)r * C);
+        }
+    }
 }
 
 inline unsigned blocks_for(long long units, int per_block) { return (unsigned)((units + per_block - 1) / per_block); }
@@ -334,22 +395,26 @@ int launch_rmsnorm_x(int x_dtype, const void* g_out, const void* x, const void* 
     }
 }
 
+template <typename T, int VEC>
+int launch_gated_as(const void* g, const void* fc1, void* out, long long n_rows, int P, int T_len, int hidden,
+                    hipStream_t stream) {
+    const long long units = n_rows * (hidden / VEC);
+    if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many elements");
+    hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, VEC>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
+                       (const T*)g, (const T*)fc1, (T*)out, units, P, T_len, hidden);
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
 template <typename T>
 int launch_gated(const void* g, const void* fc1, void* out, long long n_rows, int P, int T_len, int hidden,
                  hipStream_t stream) {
-    if (hidden % 4 == 0) {
-        const long long units = n_rows * (hidden / 4);
-        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many elements");
-        hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, 4>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
-                           (const T*)g, (const T*)fc1, (T*)out, units, P, T_len, hidden);
-    } else {
-        const long long units = n_rows * hidden;
-        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many elements");
-        hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, 1>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
-                           (const T*)g, (const T*)fc1, (T*)out, units, P, T_len, hidden);
-    }
-    LBI_HIP_CHECK(hipGetLastError());
-    return LBI_OK;
+    constexpr int W = wide<T>();
+    const bool aligned =
+        (reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(fc1) | reinterpret_cast<uintptr_t>(out)) % 16 == 0;
+    if (hidden % W == 0 && aligned) return launch_gated_as<T, W>(g, fc1, out, n_rows, P, T_len, hidden, stream);
+    if (hidden % 4 == 0 && sizeof(T) == 4) return launch_gated_as<T, 4>(g, fc1, out, n_rows, P, T_len, hidden, stream);
+    return launch_gated_as<T, 1>(g, fc1, out, n_rows, P, T_len, hidden, stream);
 }
 
 template <typename T>
@@ -373,22 +438,30 @@ int launch_qkv(const void* dq, const void* dk, const void* dv, const float* cos_
     return LBI_OK;
 }
 
-template <typename T>
-int launch_conv(const void* g_out, const void* weight, void* g_in, long long n_rows, int T_len, int C, int ksize,
-                hipStream_t stream) {
-    if (C % 4 == 0) {
-        const long long units = n_rows * (C / 4);
-        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_causal_conv1d_pullback: too many elements");
-        hipLaunchKernelGGL((causal_conv1d_pullback_kernel<T, 4>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
-                           (const T*)g_out, (const T*)weight, (T*)g_in, units, T_len, C, ksize);
-    } else {
-        const long long units = n_rows * C;
-        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_causal_conv1d_pullback: too many elements");
-        hipLaunchKernelGGL((causal_conv1d_pullback_kernel<T, 1>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
-                           (const T*)g_out, (const T*)weight, (T*)g_in, units, T_len, C, ksize);
-    }
+template <typename T, int VEC, int KMAX, int RUN>
+int launch_conv_as(const void* g_out, const void* weight, void* g_in, long long n_seq, int T_len, int C, int ksize,
+                   hipStream_t stream) {
+    const long long units = n_seq * ((T_len + RUN - 1) / RUN) * (C / VEC);
+    if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_causal_conv1d_pullback: too many elements");
+    hipLaunchKernelGGL((causal_conv1d_pullback_kernel<T, VEC, KMAX, RUN>), dim3(blocks_for(units, 256)), dim3(256), 0,
+                       stream, (const T*)g_out, (const T*)weight, (T*)g_in, units, T_len, C, ksize);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
+}
+
+template <typename T>
+int launch_conv(const void* g_out, const void* weight, void* g_in, long long n_seq, int T_len, int C, int ksize,
+                hipStream_t stream) {
+    constexpr int W = wide<T>();
+    const bool aligned = (reinterpret_cast<uintptr_t>(g_out) | reinterpret_cast<uintptr_t>(g_in)) % 16 == 0;
+    if (C % W == 0 && aligned) {
+        if (ksize <= 4) return launch_conv_as<T, W, 4, 16>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
+        if (ksize <= 8) return launch_conv_as<T, W, 8, 8>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
+    }
+    if (ksize <= 4) return launch_conv_as<T, 1, 4, 8>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
+    if (ksize <= 8) return launch_conv_as<T, 1, 8, 8>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
+    if (ksize <= 16) return launch_conv_as<T, 1, 16, 4>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
+    return launch_conv_as<T, 1, 64, 1>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
 }
 
 inline bool valid_dtype(int dtype) { return dtype == LBI_F32 || dtype == LBI_F16 || dtype == LBI_BF16; }
@@ -504,12 +577,11 @@ extern "C" int lbi_causal_conv1d_pullback(const void* g_out, const void* weight,
     if (!region::valid_dtype(dtype)) return fail(LBI_ERR_INVALID, "lbi_causal_conv1d_pullback: bad dtype %d", dtype);
     if (N < 0 || !region::positive_int(T) || !region::positive_int(C) || ksize < 1 || ksize > 64)
         return fail(LBI_ERR_INVALID, "lbi_causal_conv1d_pullback: bad size");
-    const long long n_rows = (long long)N * T;
-    if (n_rows == 0) return LBI_OK;
+    if (N == 0) return LBI_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
-        case LBI_F32: return region::launch_conv<float>(g_out, weight, g_in, n_rows, (int)T, (int)C, (int)ksize, s);
-        case LBI_F16: return region::launch_conv<_Float16>(g_out, weight, g_in, n_rows, (int)T, (int)C, (int)ksize, s);
-        default: return region::launch_conv<bf16_raw>(g_out, weight, g_in, n_rows, (int)T, (int)C, (int)ksize, s);
+        case LBI_F32: return region::launch_conv<float>(g_out, weight, g_in, N, (int)T, (int)C, (int)ksize, s);
+        case LBI_F16: return region::launch_conv<_Float16>(g_out, weight, g_in, N, (int)T, (int)C, (int)ksize, s);
+        default: return region::launch_conv<bf16_raw>(g_out, weight, g_in, N, (int)T, (int)C, (int)ksize, s);
     }
 }

@@ -158,11 +158,12 @@ def causal_conv1d_pullback(g_out: torch.Tensor, weight: torch.Tensor) -> torch.T
 
 
 def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor | None, g_residual: torch.Tensor,
-                          kernel_mode: str) -> torch.Tensor:
+                          kernel_mode: str, want_branch: bool) -> tuple[torch.Tensor, torch.Tensor | None]:
     """One block, backwards.  ``g_residual`` (fp32, [B,P,T,D]) is the cotangent of the block's
     residual output and is updated in place; ``g_hidden`` is the cotangent of its hidden output
     in the weight dtype (``None``: equal to ``g_residual``).  Returns the cotangent of
-    ``hidden (+ residual)`` at the block input, fp32."""
+    ``hidden (+ residual)`` at the block input in fp32 and, if ``want_branch``, also rounded to
+    the weight dtype (the ``g_hidden`` of the block before)."""
     attn, mlp = block.attn, block.mlp
     wdtype = mlp.fc2.weight.dtype
     a_cache, m_cache = layer_cache.attention, layer_cache.mlp
@@ -196,9 +197,8 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
         g_qkv = causal_conv1d_pullback(g_qkv, attn.conv1d.weight)
     g_norm1 = torch.matmul(g_qkv, attn.in_proj.weight)
     del g_qkv
-    g_res1, _ = rmsnorm_pullback(g_norm1, a_cache.norm_input, block.norm.weight, block.norm.eps, g_res2,
-                                 want_branch=False)
-    return g_res1
+    return rmsnorm_pullback(g_norm1, a_cache.norm_input, block.norm.weight, block.norm.eps, g_res2,
+                            want_branch=want_branch)
 
 
 def region_input_pullback_basis(backend: Any, cache: Any, output_cotangent_basis: torch.Tensor, *,
@@ -220,11 +220,13 @@ def region_input_pullback_basis(backend: Any, cache: Any, output_cotangent_basis
     device = cache.region_input.device
     # region_output = hidden + residual of the last block: both receive the cotangent
     g = output_cotangent_basis.to(device=device, dtype=torch.float32, copy=True).contiguous()
+    g_branch = None
     for offset in range(end - start - 1, -1, -1):
         layer_cache = cache.layer_caches[offset]
         block = backend.backbone.blocks[layer_cache.layer_index]
-        g = _layer_input_pullback(block, layer_cache, None, g, kernel_mode)
-        # hidden and residual at the block input enter only through their sum
+        # hidden and residual at a block input enter only through their sum, so one cotangent
+        # (fp32, and its rounded copy for the first product of the block before) is carried
+        g, g_branch = _layer_input_pullback(block, layer_cache, g_branch, g, kernel_mode, want_branch=offset > 0)
     return g.to(device=output_cotangent_basis.device, dtype=output_cotangent_basis.dtype)
 
 
