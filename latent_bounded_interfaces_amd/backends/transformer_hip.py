@@ -11,7 +11,7 @@ from typing import Any
 import torch
 
 from ..hip.transformer import attention_input_pullback_basis as hip_attention_input_pullback_basis
-from ..hip.transformer.region import region_input_pullback_basis
+from ..hip.transformer.region import region_input_pullback_basis, region_parameter_vjp
 
 
 class HipTransformerLowering:
@@ -21,9 +21,8 @@ class HipTransformerLowering:
 
     def __init__(self, *, reference_lowering: Any | None = None) -> None:
         # The reference's class can delegate the region-level methods to its autograd lowering
-        # (allow_reference_fallback=True).  Here input_pullback_basis always runs the HIP path;
-        # parameter_vjp is delegated to `reference_lowering` when one is given and raises
-        # otherwise, as the reference does by default.
+        # (allow_reference_fallback=True).  Here both run the HIP path; a caller who passes a
+        # `reference_lowering` gets parameter_vjp from it instead.
         self.reference_lowering = reference_lowering
         self.allow_reference_fallback = reference_lowering is not None
 
@@ -64,9 +63,9 @@ class HipTransformerLowering:
         return region_input_pullback_basis(backend, cache, output_cotangent_basis, kernel_mode="hip")
 
     def parameter_vjp(self, *, backend: Any, cache: Any, output_cotangent: torch.Tensor) -> dict[str, torch.Tensor]:
-        # reference backends/transformer_cuda.py:66-83
+        """Parameter gradients of the region for ``output_cotangent [B, T, D]`` on the GPU, keyed
+        like ``backend.named_parameters()`` (reference backends/transformer_cuda.py:66-83 leaves
+        this unimplemented; autograd version backends/transformer.py:332-355)."""
         if self.reference_lowering is not None:
             return self.reference_lowering.parameter_vjp(backend=backend, cache=cache, output_cotangent=output_cotangent)
-        raise NotImplementedError(
-            "HipTransformerLowering.parameter_vjp is not implemented; pass reference_lowering=... to delegate it."
-        )
+        return region_parameter_vjp(backend, cache, output_cotangent, kernel_mode="hip")

@@ -157,13 +157,59 @@ def causal_conv1d_pullback(g_out: torch.Tensor, weight: torch.Tensor) -> torch.T
     return out
 
 
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    return t.reshape(-1, t.shape[-1])
+
+
+def _linear_grads(sink: dict, linear: Any, g_out: torch.Tensor, x: torch.Tensor) -> None:
+    """Weight (and bias) gradient of ``y = x W^T + b`` for the single direction in ``g_out [B,1,T,O]``."""
+    g2 = _rows(g_out)
+    sink[id(linear.weight)] = torch.matmul(g2.t(), _rows(x).to(g2.dtype)).to(linear.weight.dtype)
+    bias = getattr(linear, "bias", None)
+    if bias is not None:
+        sink[id(bias)] = g2.float().sum(dim=0).to(bias.dtype)
+
+
+def _norm_weight_grad(sink: dict, norm: Any, g_out: torch.Tensor, x: torch.Tensor) -> None:
+    """Gradient of the RMSNorm weight: sum over rows of g_out o normalised(x), with x rounded to
+    the weight dtype first and the normalised value rounded again, as the forward does
+    (reference backbones/transformer/block.py:18-23)."""
+    wdtype = norm.weight.dtype
+    xf = x.to(wdtype).float()
+    normed = (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + norm.eps)).to(wdtype).float()
+    sink[id(norm.weight)] = (_rows(g_out).float() * _rows(normed)).sum(dim=0).to(wdtype)
+
+
+def _conv_grads(sink: dict, conv: Any, g_out: torch.Tensor, x_pre: torch.Tensor) -> None:
+    """Depthwise causal convolution: g_w[c, j] = sum_{b,t} g_out[b,t,c] x_pre[b, t + j - (k-1), c]."""
+    ksize = conv.weight.shape[-1]
+    g = g_out[:, 0].float()
+    x = x_pre.float()
+    seqlen = g.shape[1]
+    cols = []
+    for j in range(ksize):
+        shift = ksize - 1 - j
+        if shift >= seqlen:
+            cols.append(torch.zeros(g.shape[-1], device=g.device))
+        else:
+            cols.append((g[:, shift:] * x[:, :seqlen - shift]).sum(dim=(0, 1)))
+    sink[id(conv.weight)] = torch.stack(cols, dim=-1).unsqueeze(1).to(conv.weight.dtype)
+    if getattr(conv, "bias", None) is not None:
+        sink[id(conv.bias)] = g.sum(dim=(0, 1)).to(conv.bias.dtype)
+
+
 def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor | None, g_residual: torch.Tensor,
-                          kernel_mode: str, want_branch: bool) -> tuple[torch.Tensor, torch.Tensor | None]:
+                          kernel_mode: str, want_branch: bool,
+                          param_grads: dict | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
     """One block, backwards.  ``g_residual`` (fp32, [B,P,T,D]) is the cotangent of the block's
     residual output and is updated in place; ``g_hidden`` is the cotangent of its hidden output
     in the weight dtype (``None``: equal to ``g_residual``).  Returns the cotangent of
     ``hidden (+ residual)`` at the block input in fp32 and, if ``want_branch``, also rounded to
-    the weight dtype (the ``g_hidden`` of the block before)."""
+    the weight dtype (the ``g_hidden`` of the block before).
+
+    With ``param_grads`` (a dict filled as ``id(parameter) -> gradient``; P must be 1) the
+    parameter gradients of the block are formed on the way, each from the cotangent at the
+    output of its module and the cached input of that module."""
     attn, mlp = block.attn, block.mlp
     wdtype = mlp.fc2.weight.dtype
     a_cache, m_cache = layer_cache.attention, layer_cache.mlp
@@ -171,17 +217,25 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
         g_hidden = g_residual.to(wdtype)
 
     # gated MLP: hidden_out = fc2(up * silu(gate)), [up | gate] = fc1(norm2(res2))
+    if param_grads is not None:
+        _linear_grads(param_grads, mlp.fc2, g_hidden, m_cache.down_input)
     g_down_input = torch.matmul(g_hidden, mlp.fc2.weight)
     g_fc1 = gated_mlp_pullback(g_down_input, m_cache.fc1_output)
     del g_down_input
+    if param_grads is not None:
+        _linear_grads(param_grads, mlp.fc1, g_fc1, m_cache.norm_output)
     g_norm2 = torch.matmul(g_fc1, mlp.fc1.weight)
     del g_fc1
+    if param_grads is not None:
+        _norm_weight_grad(param_grads, block.norm2, g_norm2, m_cache.norm_input)
     # res2 feeds norm2 and the residual output
     g_res2, g_attn_out = rmsnorm_pullback(g_norm2, m_cache.norm_input, block.norm2.weight, block.norm2.eps,
                                           g_residual, want_branch=True)
     del g_norm2
 
     # attention: res2 = out_proj(heads) + res1
+    if param_grads is not None:
+        _linear_grads(param_grads, attn.out_proj, g_attn_out, a_cache.out_proj_input)
     g_merged = torch.matmul(g_attn_out, attn.out_proj.weight)
     del g_attn_out
     g_heads = attn_heads_split(g_merged, attn.n_heads, attn.head_dim)
@@ -194,11 +248,38 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
                               rope_interleaved=attn.rope_interleaved)
     del dq, dk, dv
     if attn.d_conv > 0:
+        if param_grads is not None:
+            # the cache keeps the projection after the convolution only: redo the projection
+            bias = getattr(attn.in_proj, "bias", None)
+            x_pre = torch.nn.functional.linear(a_cache.norm_output, attn.in_proj.weight, bias)
+            _conv_grads(param_grads, attn.conv1d, g_qkv, x_pre)
+            del x_pre
         g_qkv = causal_conv1d_pullback(g_qkv, attn.conv1d.weight)
+    if param_grads is not None:
+        _linear_grads(param_grads, attn.in_proj, g_qkv, a_cache.norm_output)
     g_norm1 = torch.matmul(g_qkv, attn.in_proj.weight)
     del g_qkv
+    if param_grads is not None:
+        _norm_weight_grad(param_grads, block.norm, g_norm1, a_cache.norm_input)
     return rmsnorm_pullback(g_norm1, a_cache.norm_input, block.norm.weight, block.norm.eps, g_res2,
                             want_branch=want_branch)
+
+
+def _pull_back_region(backend: Any, cache: Any, cotangent: torch.Tensor, kernel_mode: str,
+                      param_grads: dict | None) -> torch.Tensor:
+    start, end = cache.layer_range
+    device = cache.region_input.device
+    # region_output = hidden + residual of the last block: both receive the cotangent
+    g = cotangent.to(device=device, dtype=torch.float32, copy=True).contiguous()
+    g_branch = None
+    for offset in range(end - start - 1, -1, -1):
+        layer_cache = cache.layer_caches[offset]
+        block = backend.backbone.blocks[layer_cache.layer_index]
+        # hidden and residual at a block input enter only through their sum, so one cotangent
+        # (fp32, and its rounded copy for the first product of the block before) is carried
+        g, g_branch = _layer_input_pullback(block, layer_cache, g_branch, g, kernel_mode, want_branch=offset > 0,
+                                            param_grads=param_grads)
+    return g
 
 
 def region_input_pullback_basis(backend: Any, cache: Any, output_cotangent_basis: torch.Tensor, *,
@@ -217,20 +298,41 @@ def region_input_pullback_basis(backend: Any, cache: Any, output_cotangent_basis
         raise ValueError("cache.layer_caches does not match cache.layer_range")
     if end == start:
         return output_cotangent_basis.clone()
-    device = cache.region_input.device
-    # region_output = hidden + residual of the last block: both receive the cotangent
-    g = output_cotangent_basis.to(device=device, dtype=torch.float32, copy=True).contiguous()
-    g_branch = None
-    for offset in range(end - start - 1, -1, -1):
-        layer_cache = cache.layer_caches[offset]
-        block = backend.backbone.blocks[layer_cache.layer_index]
-        # hidden and residual at a block input enter only through their sum, so one cotangent
-        # (fp32, and its rounded copy for the first product of the block before) is carried
-        g, g_branch = _layer_input_pullback(block, layer_cache, g_branch, g, kernel_mode, want_branch=offset > 0)
+    g = _pull_back_region(backend, cache, output_cotangent_basis, kernel_mode, None)
     return g.to(device=output_cotangent_basis.device, dtype=output_cotangent_basis.dtype)
+
+
+def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tensor, *,
+                         kernel_mode: str = "hip") -> dict[str, torch.Tensor]:
+    """Parameter gradients of one region for ``output_cotangent [B, T, D]``, keyed by the
+    parameter names of ``backend.named_parameters()``.
+
+    ``TransformerLowering.parameter_vjp`` of the reference (backends/transformer.py:76-85;
+    autograd version :332-355).  One backward sweep over the cached activations with a single
+    direction; every weight gradient is a plain GEMM of the cotangent at a module's output
+    with the module's cached input.
+    """
+    if output_cotangent.dim() != 3:
+        raise ValueError("output_cotangent must have shape [B, T, D]")
+    if not output_cotangent.is_cuda:
+        raise RuntimeError("output_cotangent must be a CUDA tensor (this build has no CPU execution path)")
+    start, end = cache.layer_range
+    if len(cache.layer_caches) != end - start:
+        raise ValueError("cache.layer_caches does not match cache.layer_range")
+    by_id: dict[int, torch.Tensor] = {}
+    if end > start:
+        with torch.no_grad():
+            _pull_back_region(backend, cache, output_cotangent.unsqueeze(1), kernel_mode, by_id)
+    wanted = {id(p) for layer_cache in cache.layer_caches
+              for p in backend.backbone.blocks[layer_cache.layer_index].parameters() if p.requires_grad}
+    out: dict[str, torch.Tensor] = {}
+    for name, param in backend.named_parameters():
+        if id(param) in wanted and id(param) in by_id:
+            out[name] = by_id[id(param)].detach()
+    return out
 
 
 __all__ = [
     "attn_heads_split", "attn_qkv_pullback", "causal_conv1d_pullback", "gated_mlp_pullback", "rmsnorm_pullback",
-    "region_input_pullback_basis", "rope_tables",
+    "region_input_pullback_basis", "region_parameter_vjp", "rope_tables",
 ]

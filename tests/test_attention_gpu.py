@@ -127,8 +127,10 @@ def test_modes_and_contract(device):
         low.input_pullback_basis(backend=None, cache=None, output_cotangent_basis=torch.zeros(1, 1, 2, 3))
     with pytest.raises(ValueError):
         low.input_pullback_basis(backend=None, cache=None, output_cotangent_basis=torch.zeros(1, 2, 3))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="no CPU execution path"):
         low.parameter_vjp(backend=None, cache=None, output_cotangent=torch.zeros(1, 2, 3))
+    with pytest.raises(ValueError):
+        low.parameter_vjp(backend=None, cache=None, output_cotangent=torch.zeros(1, 2, 3, 4))
 
 
 def test_long_context_properties(device):

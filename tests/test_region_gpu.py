@@ -217,3 +217,55 @@ def test_region_pullback_contract(device):
     # a zero-layer range is the identity
     cache.layer_range, cache.layer_caches = (0, 0), []
     assert torch.equal(low.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=basis), basis)
+
+
+@pytest.mark.parametrize("case", REGION_CASES)
+@pytest.mark.parametrize("bias", [False, True])
+def test_parameter_vjp_fp32_matches_autograd(case, bias, device):
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+
+    dim, heads, kv, hd, hidden, layers, d_conv, inter, b, p, t = case
+    backend = oreg.make_backend(dim=dim, n_heads=heads, n_kv_heads=kv, head_dim=hd, hidden=hidden, layers=layers + 1,
+                                region_ranges=[(0, 1), (1, layers + 1)], d_conv=d_conv, rope_interleaved=inter,
+                                rope_base=1000.0, bias=bias, seed=dim + 1)
+    torch.manual_seed(t)
+    x = torch.randn(b, t, dim)
+    cot = torch.randn(b, t, dim)
+    _, cpu_cache = backend.forward_region(region_input=x, region_index=1)
+    want = oreg.parameter_vjp_autograd(backend, cpu_cache, cot)
+
+    gpu_backend = backend.to(device)
+    with torch.no_grad():
+        _, cache = gpu_backend.forward_region(region_input=x.to(device), region_index=1)
+    got = HipTransformerLowering().parameter_vjp(backend=gpu_backend, cache=cache, output_cotangent=cot.to(device))
+    assert set(got) == set(want) and all(n.startswith("backbone.blocks.") for n in got)
+    assert not any(n.startswith("backbone.blocks.0.") for n in got)  # region 1 owns layers 1..
+    for name, w in want.items():
+        g = got[name].cpu()
+        assert g.shape == w.shape and g.dtype == w.dtype
+        assert _max_rel(g, w) <= 2e-5, (name, _max_rel(g, w))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_parameter_vjp_16bit_matches_fp32_path(dtype, device):
+    import copy
+
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+
+    dim, heads, kv, hd, hidden, layers, b, t = 128, 2, 1, 64, 256, 2, 2, 128
+    backend = oreg.make_backend(dim=dim, n_heads=heads, n_kv_heads=kv, head_dim=hd, hidden=hidden, layers=layers,
+                                d_conv=4, dtype=dtype, seed=13)
+    torch.manual_seed(14)
+    x = torch.randn(b, t, dim).to(dtype)
+    cot = torch.randn(b, t, dim)
+    ref_backend = copy.deepcopy(backend).float()
+    _, ref_cache = ref_backend.forward_region(region_input=x.float(), region_index=0)
+    want = oreg.parameter_vjp_autograd(ref_backend, ref_cache, cot)
+    gpu_backend = backend.to(device)
+    with torch.no_grad():
+        _, cache = gpu_backend.forward_region(region_input=x.to(device), region_index=0)
+    got = HipTransformerLowering().parameter_vjp(backend=gpu_backend, cache=cache, output_cotangent=cot.to(device))
+    assert set(got) == set(want)
+    for name, w in want.items():
+        assert got[name].dtype == dtype
+        assert _max_rel(got[name].cpu(), w) <= 3e-2, (name, _max_rel(got[name].cpu(), w))
