@@ -14,7 +14,8 @@ Prints ONE JSON line.  Besides the contract keys it carries
 * ``cpu_baseline``  - the reference's CPU algorithm (log-depth torch scan) timed on the
                       host cores of the same box on a bounded batch slice;
 * ``extra``         - the other measured variants (bf16 storage, cotangent-only chain,
-                      attention input-pullback) with their own roofline figures.
+                      attention input-pullback, region-level input pullback) with their own
+                      roofline figures.
 """
 from __future__ import annotations
 
@@ -239,6 +240,8 @@ def main() -> int:
             from latent_bounded_interfaces_amd import benchmarks as lbi_bench
 
             extra.update(lbi_bench.attention_section(steps=max(3, args.steps // 4)))
+            torch.cuda.empty_cache()
+            extra.update(lbi_bench.region_section(steps=max(3, args.steps // 4)))
         except ImportError:
             pass
         result["extra"] = extra
