@@ -37,6 +37,14 @@ __device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned 
                  : "memory");
 }
 
+// The same with a full 64-bit address per lane (no common base).
+__device__ __forceinline__ void dma16_at(const void* lane_ptr, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(lane_ptr)
+                 : "memory");
+}
+
 template <typename T, int DH, bool CAUSAL>
 __global__ __launch_bounds__(256) void dkdv_ring_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                       const T* __restrict__ v, const T* __restrict__ d_out,
@@ -89,9 +97,9 @@ __global__ __launch_bounds__(256) void dkdv_ring_kernel(const T* __restrict__ q,
         const int r = sigma / CPR;
         dma_off[x] = r * RB + (((sigma % CPR) ^ swz<DH>(r)) << 4);
     }
-    // lanes 0-7: lse2 float4 #lane, lanes 8-15: delta float4 #(lane-8), as offsets from lse_bh
-    const unsigned stat_off =
-        (lane < 8 ? 0u : (unsigned)((const char*)delta_p - (const char*)lse_bh)) + 16 * (lane & 7);
+    // lanes 0-7: lse2 float4 #lane, lanes 8-15: delta float4 #(lane-8); the two arrays need not
+    // share an allocation, so each lane carries its own 64-bit address
+    const float* stat_ptr = (lane < 8 ? lse_bh : delta_p) + 4 * (lane & 7);
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char*)smem;
     auto issue_tile = [&](int i_row, unsigned stage_base) __attribute__((always_inline)) {
         const unsigned row_bytes = (unsigned)i_row * RB;
@@ -101,7 +109,7 @@ __global__ __launch_bounds__(256) void dkdv_ring_kernel(const T* __restrict__ q,
             dma16(g_p, row_bytes + dma_off[x], lds0 + stage_base + TILE + 1024 * (NX * wave + x));
         }
         // Every wave keeps its own copy of the 64 row statistics: no cross-wave dependency.
-        if (lane < 16) dma16(lse_bh, (unsigned)i_row * 4 + stat_off, lds0 + stage_base + 2 * TILE + 256 * wave);
+        if (lane < 16) dma16_at(stat_ptr + i_row, lds0 + stage_base + 2 * TILE + 256 * wave);
     };
 
     // K of this wave's 64 keys stays in registers (B operand of S).  V of the same keys sits
