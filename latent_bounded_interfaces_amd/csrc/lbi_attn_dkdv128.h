@@ -142,10 +142,6 @@ __global__ __launch_bounds__(256) void dkdv_ring_kernel(const T* __restrict__ q,
         }
     const float sc2 = scale * LOG2E;
 
-    // One tile step on the stage at byte offset SB.  thr: element (t, 8g+e) is above the
-    // diagonal iff 8g + e < thr + 32t.
-    // LDS operand reads are written a block ahead of their use so their latency can pass
-    // under the products of the block before.
     auto lds16 = [&](const char* p) __attribute__((always_inline)) {
         return *reinterpret_cast<const u32x4*>(p);
     };
@@ -162,111 +158,172 @@ __global__ __launch_bounds__(256) void dkdv_ring_kernel(const T* __restrict__ q,
         return u32x4{l2[0], l2[1], h2[0], h2[1]};
     };
 
-    // One tile step on the stage at byte offset SB.  thr: element (t, 8g+e) is above the
-    // diagonal iff 8g + e < thr + 32t.
-    auto step = [&](auto mask_tag, auto stage_tag, int thr) __attribute__((always_inline)) {
+    // One tile step on the stage at byte offset SB: 8 KS matrix products in four phases,
+    //   S = Q K^T   dP = dO V^T - delta   dV += P^T dO   dK += dS^T Q        (2 KS, 2 KS, 4 ND, 4 ND products)
+    // and sixteen "quanta" of vector work, one per (g, t) block of four rows of a 32 x 32 tile:
+    //   P quantum:  exp2(S c - lse2), mask, round, pack        dS quantum:  P o dP, round, pack
+    // The matrix pipe overlaps vector instructions of the same wave only while few of them sit
+    // between two products, so the quanta are spread thinly over the products that do not
+    // need their results yet instead of being bunched behind the phase that feeds them:
+    //   P quanta 0-3 (rows 0-15: the k-step 0 operands of dV) under the dP products, 4-7 under
+    //   the first half of dV; dS quanta 0-3 under the second half of dV, 4-7 under the first
+    //   half of dK.  LDS operands are fetched two product pairs ahead of their use.
+    // thr: element (t, 8g+e) is above the diagonal iff 8g + e < thr + 32t.
+    // Operands of the S phase and the row statistics of the step to come: fetched during the
+    // dK phase of the step before (the first ones ahead of the loop), so a step starts with
+    // its products, not with LDS latency.
+    u32x4 qa[KS];
+    f32x4 lq[4];      // lse2 of rows 8g + 4h .. + 3
+    f32x16 nd16;      // -delta of the same rows, laid out as an accumulator tile
+    auto fetch_q = [&](const char* stage, int ks) __attribute__((always_inline)) {
+        qa[ks] = lds16(stage + (lane_nat ^ (ks << 5)));
+    };
+    auto fetch_stats = [&](const char* stage, int g) __attribute__((always_inline)) {
+        lq[g] = lds_f4(stage + 2 * TILE + lane_stat + 32 * g);
+        const f32x4 d4 = lds_f4(stage + 2 * TILE + lane_stat + 128 + 32 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) nd16[4 * g + e] = d4[e];
+    };
+
+    auto step = [&](auto mask_tag, auto stage_tag, auto next_tag, auto refill_tag, int thr, int refill_row)
+                    __attribute__((always_inline)) {
         constexpr bool MASK = decltype(mask_tag)::value;
         constexpr unsigned SB = decltype(stage_tag)::value;
+        constexpr unsigned SN = decltype(next_tag)::value;      // stage of the next tile
+        constexpr unsigned SR = decltype(refill_tag)::value;    // stage of the tile before: free after the mid-step barrier
+        constexpr int NS = 2 * KS;      // products of the S phase (and of the dP phase)
+        constexpr int NA = 4 * ND;      // products of the dV phase (and of the dK phase)
+        constexpr int NPROD = 2 * NS + 2 * NA;
         const char* qt = smem + SB;
         const char* gt = smem + SB + TILE;
         const char* st = smem + SB + 2 * TILE;
 
-        // ---- S = Q K^T: all eight Q fragments in flight at once, then the first dP operands.
-        u32x4 qa[KS];
+        u32x4 ga[3], va[3], vb[3];  // dP operands of k-step ks live in slot ks % 3
+        auto fetch_dp = [&](int ks) __attribute__((always_inline)) {
+            ga[ks % 3] = lds16(gt + (lane_nat ^ (ks << 5)));
+            va[ks % 3] = lds16(vt + (lane_nat ^ (ks << 5)));
+            vb[ks % 3] = lds16(vt + TILE + (lane_nat ^ (ks << 5)));
+        };
+        u32x4 bfr[3];  // tr fragment f of the dV (f < 2 ND: d_out tile) and dK (Q tile) phases lives in slot f % 3
+        auto fetch_tr = [&](int f) __attribute__((always_inline)) {
+            if (f < 2 * ND) bfr[f % 3] = tr_frag(gt, f / ND, f % ND);
+            else if (f < 4 * ND) bfr[f % 3] = tr_frag(qt, (f - 2 * ND) / ND, (f - 2 * ND) % ND);
+        };
+        f32x16 s[2], dp[2];
+        u32x4 pa[2][2], dsa[2][2];
+
+        auto p_quantum = [&](int q) __attribute__((always_inline)) {
+            const int g = q >> 1, t = q & 1;
+            pin_tile(s[t]);
+            float pr[4];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qa[ks] = lds16(qt + (lane_nat ^ (ks << 5)));
-        u32x4 ga[2], va[2], vb[2];  // dP operands of block ks live in slot ks & 1
-        ga[0] = lds16(gt + lane_nat);
-        va[0] = lds16(vt + lane_nat);
-        vb[0] = lds16(vt + TILE + lane_nat);
-        f32x16 s[2];
+            for (int e = 0; e < 4; ++e) {
+                pr[e] = __builtin_amdgcn_exp2f(s[t][4 * g + e] * sc2 - lq[g][e]);
+                if (MASK && (8 * g + e < thr + 32 * t)) pr[e] = 0.0f;
+            }
+            unsigned w0 = Mma<T>::pack2(pr[0], pr[1]), w1 = Mma<T>::pack2(pr[2], pr[3]);
+            pin_here(w0, w1);
+            pa[t][g >> 1][2 * (g & 1)] = w0;
+            pa[t][g >> 1][2 * (g & 1) + 1] = w1;
+        };
+        auto ds_quantum = [&](int q) __attribute__((always_inline)) {
+            const int g = q >> 1, t = q & 1;
+            pin_tile(dp[t]);
+            const unsigned p0 = pa[t][g >> 1][2 * (g & 1)], p1 = pa[t][g >> 1][2 * (g & 1) + 1];
+            const float d0 = Mma<T>::lo(p0) * dp[t][4 * g + 0];  // dp already holds dP - delta
+            const float d1 = Mma<T>::hi(p0) * dp[t][4 * g + 1];
+            const float d2 = Mma<T>::lo(p1) * dp[t][4 * g + 2];
+            const float d3 = Mma<T>::hi(p1) * dp[t][4 * g + 3];
+            unsigned w0 = Mma<T>::pack2(d0, d1), w1 = Mma<T>::pack2(d2, d3);
+            pin_here(w0, w1);
+            dsa[t][g >> 1][2 * (g & 1)] = w0;
+            dsa[t][g >> 1][2 * (g & 1) + 1] = w1;
+        };
+        // Vector work and LDS fetches slotted after product i (0-based over the whole step).
+        auto after = [&](int i) __attribute__((always_inline)) {
+            __builtin_amdgcn_sched_barrier(0);  // nothing moves across a product: the slotting below is the schedule
+            // ---- fetches
+            if (i == NS / 2) fetch_dp(0);
+            if (i == NS / 2 + 2) fetch_dp(1);
+            if (i == NS - 2) fetch_dp(2);
+            if (i >= NS && i < 2 * NS && (i & 1)) {            // pair ks = (i - NS) / 2 consumed: refill its slot
+                const int ks = (i - NS) / 2;
+                if (ks + 3 < KS) fetch_dp(ks + 3);
+            }
+            if (i == 2 * NS - 6) fetch_tr(0);
+            if (i == 2 * NS - 4) fetch_tr(1);
+            if (i == 2 * NS - 2) fetch_tr(2);
+            if (i >= 2 * NS && (i & 1)) fetch_tr((i - 2 * NS) / 2 + 3);  // fragment (i - 2NS)/2 consumed
+            if (i == 2 * NS - 1) {
+                // Half way: this wave's share of the next tile has landed once all but the newest
+                // tile load is done; the barrier publishes everyone's share and tells that every wave
+                // is done with the tile before this one, whose stage is refilled.  (No LDS wait: the
+                // reads in flight belong to stages that stay as they are.)
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm((R - 3) * NDMA));
+                __builtin_amdgcn_s_barrier();
+                issue_tile(refill_row, SR);
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                if (i == 2 * NS + NA + 2 * ks) fetch_q(smem + SN, ks);
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                if (i == 2 * NS + NA + 1 + 2 * g) fetch_stats(smem + SN, g);
+            // ---- quanta.  Sixteen quanta over the products NS+1 .. NPROD-NA/2-2, evenly.
+            constexpr int first = NS + 1, span = NPROD - NA / 2 - 2 - first;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                if (i == first + (q * span) / 15) {
+                    if (q == 0) mma_v_settle(s[0], s[1]);
+                    if (q < 8) p_quantum(q);
+                    else ds_quantum(q - 8);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+
+        // ---- S = Q K^T
         s[0] = Mma<T>::mma_v_start(qa[0], kf[0][0]);
+        after(0);
         s[1] = Mma<T>::mma_v_start(qa[0], kf[1][0]);
+        after(1);
 #pragma unroll
         for (int ks = 1; ks < KS; ++ks) {
             Mma<T>::mma_v(qa[ks], kf[0][ks], s[0]);
+            after(2 * ks);
             Mma<T>::mma_v(qa[ks], kf[1][ks], s[1]);
+            after(2 * ks + 1);
         }
-        f32x4 l4 = lds_f4(st + lane_stat);
-        mma_v_settle(s[0], s[1]);
-
-        // ---- dP = dO V^T, with the P phase (exp2, mask, pack) of one (g, t) block of S after
-        // each pair of products: independent work, so it runs while the matrix pipe is busy.
-        f32x16 dp[2];
-        u32x4 pa[2][2], dsa[2][2];
+        // ---- dP - delta = dO V^T - delta
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const int cur = ks & 1, nxt = cur ^ 1;
-            if (ks + 1 < KS) {
-                ga[nxt] = lds16(gt + (lane_nat ^ ((ks + 1) << 5)));
-                va[nxt] = lds16(vt + (lane_nat ^ ((ks + 1) << 5)));
-                vb[nxt] = lds16(vt + TILE + (lane_nat ^ ((ks + 1) << 5)));
-            }
-            if (ks == 0) {
-                dp[0] = Mma<T>::mma_v_start(ga[cur], va[cur]);
-                dp[1] = Mma<T>::mma_v_start(ga[cur], vb[cur]);
+            if (ks == 0) dp[0] = Mma<T>::mma_v_c(ga[0], va[0], nd16);
+            else Mma<T>::mma_v(ga[ks % 3], va[ks % 3], dp[0]);
+            after(NS + 2 * ks);
+            if (ks == 0) dp[1] = Mma<T>::mma_v_c(ga[0], vb[0], nd16);
+            else Mma<T>::mma_v(ga[ks % 3], vb[ks % 3], dp[1]);
+            after(NS + 2 * ks + 1);
+        }
+        // ---- dV += P^T dO, then dK += dS^T Q
+#pragma unroll
+        for (int f = 0; f < 4 * ND; ++f) {
+            const int ff = f % (2 * ND), kk = ff / ND, nd = ff % ND;
+            if (f < 2 * ND) {
+                acc_v[0][nd] = Mma<T>::mma(pa[0][kk], bfr[f % 3], acc_v[0][nd]);
+                after(2 * NS + 2 * f);
+                acc_v[1][nd] = Mma<T>::mma(pa[1][kk], bfr[f % 3], acc_v[1][nd]);
+                after(2 * NS + 2 * f + 1);
             } else {
-                Mma<T>::mma_v(ga[cur], va[cur], dp[0]);
-                Mma<T>::mma_v(ga[cur], vb[cur], dp[1]);
+                acc_k[0][nd] = Mma<T>::mma(dsa[0][kk], bfr[f % 3], acc_k[0][nd]);
+                after(2 * NS + 2 * f);
+                acc_k[1][nd] = Mma<T>::mma(dsa[1][kk], bfr[f % 3], acc_k[1][nd]);
+                after(2 * NS + 2 * f + 1);
             }
-#pragma unroll
-            for (int bb = 0; bb < 8 / KS; ++bb) {  // the eight (g, t) blocks of S spread over the KS products
-                const int blk = ks * (8 / KS) + bb;
-                const int g = blk >> 1, t = blk & 1;
-                float pr[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    pr[e] = __builtin_amdgcn_exp2f(s[t][4 * g + e] * sc2 - l4[e]);
-                    if (MASK && (8 * g + e < thr + 32 * t)) pr[e] = 0.0f;
-                }
-                unsigned w0 = Mma<T>::pack2(pr[0], pr[1]), w1 = Mma<T>::pack2(pr[2], pr[3]);
-                if (t == 1 && g < 3) l4 = lds_f4(st + lane_stat + 32 * (g + 1));
-                pin_here(w0, w1);
-                pa[t][g >> 1][2 * (g & 1)] = w0;
-                pa[t][g >> 1][2 * (g & 1) + 1] = w1;
-            }
-        }
-        f32x4 d4 = lds_f4(st + lane_stat + 128);
-        u32x4 bfr[2];  // tr fragments of step i live in slot i & 1
-        bfr[0] = tr_frag(gt, 0, 0);
-        mma_v_settle(dp[0], dp[1]);
-
-        // ---- dV += P^T dO (needs P only), with the dS phase of one (g, t) block after each pair.
-#pragma unroll
-        for (int i = 0; i < 2 * ND; ++i) {
-            const int kk = i / ND, nd = i % ND, cur = i & 1;
-            bfr[cur ^ 1] = (i + 1 < 2 * ND) ? tr_frag(gt, (i + 1) / ND, (i + 1) % ND) : tr_frag(qt, 0, 0);
-            acc_v[0][nd] = Mma<T>::mma(pa[0][kk], bfr[cur], acc_v[0][nd]);
-            acc_v[1][nd] = Mma<T>::mma(pa[1][kk], bfr[cur], acc_v[1][nd]);
-#pragma unroll
-            for (int bb = 0; bb < 4 / ND; ++bb) {  // the eight (g, t) blocks of dS spread over the 2 ND steps
-                const int blk = i * (4 / ND) + bb;
-                const int g = blk >> 1, t = blk & 1;
-                const unsigned p0 = pa[t][g >> 1][2 * (g & 1)], p1 = pa[t][g >> 1][2 * (g & 1) + 1];
-                const float d0 = Mma<T>::lo(p0) * (dp[t][4 * g + 0] - d4[0]);
-                const float d1 = Mma<T>::hi(p0) * (dp[t][4 * g + 1] - d4[1]);
-                const float d2 = Mma<T>::lo(p1) * (dp[t][4 * g + 2] - d4[2]);
-                const float d3 = Mma<T>::hi(p1) * (dp[t][4 * g + 3] - d4[3]);
-                unsigned w0 = Mma<T>::pack2(d0, d1), w1 = Mma<T>::pack2(d2, d3);
-                if (t == 1 && g < 3) d4 = lds_f4(st + lane_stat + 128 + 32 * (g + 1));
-                pin_here(w0, w1);
-                dsa[t][g >> 1][2 * (g & 1)] = w0;
-                dsa[t][g >> 1][2 * (g & 1) + 1] = w1;
-            }
-        }
-
-        // ---- dK += dS^T Q
-#pragma unroll
-        for (int i = 0; i < 2 * ND; ++i) {
-            const int kk = i / ND, nd = i % ND, cur = i & 1;
-            if (i + 1 < 2 * ND) bfr[cur ^ 1] = tr_frag(qt, (i + 1) / ND, (i + 1) % ND);
-            acc_k[0][nd] = Mma<T>::mma(dsa[0][kk], bfr[cur], acc_k[0][nd]);
-            acc_k[1][nd] = Mma<T>::mma(dsa[1][kk], bfr[cur], acc_k[1][nd]);
         }
     };
 
-    // ---- tile loop: a ring of R stages filled R-1 steps ahead.  A group is R consecutive
-    // steps, so every stage offset is an immediate.  Steps past the end of the sequence
+    // ---- tile loop: a ring of R stages; tile it + R - 1 is requested half way through step it.
+    // A group is R consecutive steps, so every stage offset is an immediate.  Steps past the end of the sequence
     // (the group count is rounded up) run on a re-read tile with everything masked.
     const int i_begin = CAUSAL ? kb * 256 : 0;
     const int n_it = (T_len - i_begin) / 32;
@@ -276,16 +333,19 @@ __global__ __launch_bounds__(256) void dkdv_ring_kernel(const T* __restrict__ q,
     auto tile_row = [&](int it) __attribute__((always_inline)) { return min(i_begin + it * 32, T_len - 32); };
 #pragma unroll
     for (int x = 0; x < R - 1; ++x) issue_tile(tile_row(x), x * STAGE);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((R - 2) * NDMA));  // tile 0
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) fetch_q(smem, ks);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) fetch_stats(smem, g);
     auto one_step = [&](auto mask_tag, auto slot_tag, int it) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_tag)::value;
-        // this wave's share of tile `it` has landed once all but the newest R-2 tile loads are done;
-        // the barrier publishes everyone's share and retires the stage read in the step before.
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm((R - 2) * NDMA));
-        __syncthreads();
-        issue_tile(tile_row(it + R - 1), ((SLOT + R - 1) % R) * STAGE);
         // real steps of the non-causal case mask nothing; padding steps mask everything
         const int thr = it >= n_it ? (1 << 20) : CAUSAL ? j0w + m - 4 * h - (i_begin + it * 32) : -(1 << 20);
-        step(mask_tag, std::integral_constant<unsigned, SLOT * STAGE>{}, thr);
+        step(mask_tag, std::integral_constant<unsigned, SLOT * STAGE>{},
+             std::integral_constant<unsigned, ((SLOT + 1) % R) * STAGE>{},
+             std::integral_constant<unsigned, ((SLOT + R - 1) % R) * STAGE>{}, thr, tile_row(it + R - 1));
     };
     auto group = [&](auto mask_tag, int it0) __attribute__((always_inline)) {
         one_step(mask_tag, std::integral_constant<int, 0>{}, it0);

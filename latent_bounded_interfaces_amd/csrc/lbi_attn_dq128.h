@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void dq_ring_kernel(const T* __restrict__ q, c
     for (int pp = 0; pp < PB; ++pp) {
         const int p = min(p0 + pp, P - 1);  // surplus slots redo the last direction; never stored
         const size_t row0 = (((size_t)b * P + p) * H + hh) * T_len + i0w;
-        my_delta[pp] = delta[row0 + m];
+        my_delta[pp] = -delta[row0 + m];  // the workspace keeps -delta
 #pragma unroll
         for (int u = 0; u < CPR / 2; ++u) {
             const int slot = 64 * u + lane;

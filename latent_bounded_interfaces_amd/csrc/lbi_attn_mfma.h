@@ -4,7 +4,7 @@
 // Four kernels per call, all atomic-free (every output tile has one owner, sums run
 // in a fixed order, so reruns are bit-identical):
 //   stats_kernel  flash-style forward: lse2[b,h,i] (log2 domain) and O = softmax(..) V (fp32)
-//   delta_kernel  delta[b,p,h,i] = sum_d d_out[b,p,h,i,d] * O[b,h,i,d]
+//   delta_kernel  -delta[b,p,h,i] = -sum_d d_out[b,p,h,i,d] * O[b,h,i,d]  (kept negated in the workspace)
 //   dq_ring_kernel    owner = 32 queries per wave, PB directions at once; streams K/V tiles
 //                     (lbi_attn_dq128.h)
 //   dkdv_ring_kernel  owner = 64 keys per wave, one direction; streams Q/d_out tiles
@@ -64,6 +64,12 @@ template <> struct Mma<bf16_raw> {
     static __device__ __forceinline__ void mma_v(u32x4 a, u32x4 b, f32x16& c) {
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
     }
+    // start with C taken from another register tile (left untouched)
+    static __device__ __forceinline__ f32x16 mma_v_c(u32x4 a, u32x4 b, const f32x16& c) {
+        f32x16 d;
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+        return d;
+    }
     static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w << 16); }
     static __device__ __forceinline__ float hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
     static __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
@@ -84,6 +90,11 @@ template <> struct Mma<_Float16> {
     }
     static __device__ __forceinline__ void mma_v(u32x4 a, u32x4 b, f32x16& c) {
         asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ f32x16 mma_v_c(u32x4 a, u32x4 b, const f32x16& c) {
+        f32x16 d;
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+        return d;
     }
     static __device__ __forceinline__ float lo(unsigned w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
     static __device__ __forceinline__ float hi(unsigned w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
@@ -173,6 +184,10 @@ __device__ __forceinline__ void mma_v_settle(f32x16& c0) { asm volatile("s_nop 1
 // MFMAs are volatile too, so VALU work written between two of them stays between them
 // and runs while the matrix pipe is busy).
 __device__ __forceinline__ void pin_here(unsigned& w0, unsigned& w1) { asm volatile("" : "+v"(w0), "+v"(w1)); }
+
+// Makes every later read of the tile depend on this point of the program (no instruction
+// is emitted): work on the tile cannot be hoisted above it.
+__device__ __forceinline__ void pin_tile(f32x16& c) { asm volatile("" : "+v"(c)); }
 
 __device__ __forceinline__ f32x16 zero16() {
     f32x16 z;
@@ -330,14 +345,14 @@ __global__ __launch_bounds__(256) void delta_kernel(const T* __restrict__ d_out,
     }
 #pragma unroll
     for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, LPR);
-    if (part == 0 && row < n_rows) delta[row] = acc;
+    if (part == 0 && row < n_rows) delta[row] = -acc;  // stored negated: the dK/dV kernel starts dP from it
 }
 
 inline bool supports(int T_len, int dh, int dtype) {
     return (dtype == LBI_F16 || dtype == LBI_BF16) && (dh == 64 || dh == 128) && T_len >= 64 && T_len % 64 == 0;
 }
 
-// floats: lse2[B*H*T], delta[B*P*H*T], o32[B*H*T*Dh]
+// floats: lse2[B*H*T], -delta[B*P*H*T], o32[B*H*T*Dh]
 inline size_t workspace_floats(int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P) {
     return (size_t)(B * H * T + B * P * H * T + B * H * T * Dh);
 }
