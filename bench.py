@@ -242,6 +242,8 @@ def main() -> int:
             extra.update(lbi_bench.attention_section(steps=max(3, args.steps // 4)))
             torch.cuda.empty_cache()
             extra.update(lbi_bench.region_section(steps=max(3, args.steps // 4)))
+            torch.cuda.empty_cache()
+            extra.update(lbi_bench.lbi_step_section(steps=3))
         except ImportError:
             pass
         result["extra"] = extra

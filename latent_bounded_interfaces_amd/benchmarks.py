@@ -123,10 +123,15 @@ def attention_section(steps: int = 5) -> dict:
 # ---------------------------------------------------------------------------------------
 # Region-level input pullback (a range of Transformer layers, P cotangent directions)
 # ---------------------------------------------------------------------------------------
+class _Holder(torch.nn.Module):
+    """Parameter container with the attribute layout of the reference's Transformer block
+    (no forward: the benchmarks feed synthetic caches)."""
+
+
 def synthetic_region(*, dim, n_heads, n_kv_heads, head_dim, hidden, layers, d_conv, batch, seq_len, dtype, device,
                      residual_in_fp32=True, seed=0):
     """Random weights and a random forward cache with the attribute names of the reference's
-    ``TransformerRegionBackend`` / ``TransformerRegionCache`` (only the fields the pullback reads).
+    ``TransformerRegionBackend`` / ``TransformerRegionCache`` (the fields the pullbacks read).
     Values are synthetic (N(0,1) activations, N(0,1/fan_in) weights); shapes and dtypes are the real ones."""
     from types import SimpleNamespace as NS
 
@@ -135,25 +140,49 @@ def synthetic_region(*, dim, n_heads, n_kv_heads, head_dim, hidden, layers, d_co
     def rand(*shape, std=1.0, dt=dtype):
         return (torch.randn(*shape, generator=gen) * std).to(dt).to(device)
 
+    def linear(out_features, in_features):
+        mod = torch.nn.Linear(in_features, out_features, bias=False, device=device, dtype=dtype)
+        with torch.no_grad():
+            mod.weight.copy_(rand(out_features, in_features, std=in_features ** -0.5))
+        return mod
+
+    def norm():
+        mod = _Holder()
+        mod.weight = torch.nn.Parameter(rand(dim) * 0.1 + 1)
+        mod.eps = 1e-5
+        return mod
+
     res_dtype = torch.float32 if residual_in_fp32 else dtype
     qkv_dim = (n_heads + 2 * n_kv_heads) * head_dim
     blocks, caches = [], []
     for layer in range(layers):
-        attn = NS(n_heads=n_heads, n_kv_heads=n_kv_heads, head_dim=head_dim, rope_base=10000.0, rope_interleaved=False,
-                  softmax_scale=None, d_conv=d_conv,
-                  in_proj=NS(weight=rand(qkv_dim, dim, std=dim ** -0.5)),
-                  out_proj=NS(weight=rand(dim, n_heads * head_dim, std=(n_heads * head_dim) ** -0.5)))
+        attn = _Holder()
+        attn.n_heads, attn.n_kv_heads, attn.head_dim = n_heads, n_kv_heads, head_dim
+        attn.rope_base, attn.rope_interleaved, attn.softmax_scale, attn.d_conv = 10000.0, False, None, d_conv
+        attn.in_proj = linear(qkv_dim, dim)
+        attn.out_proj = linear(dim, n_heads * head_dim)
         if d_conv > 0:
-            attn.conv1d = NS(weight=rand(qkv_dim, 1, d_conv, std=d_conv ** -0.5))
-        mlp = NS(fc1=NS(weight=rand(2 * hidden, dim, std=dim ** -0.5)), fc2=NS(weight=rand(dim, hidden, std=hidden ** -0.5)))
-        blocks.append(NS(attn=attn, mlp=mlp, norm=NS(weight=rand(dim) * 0.1 + 1, eps=1e-5),
-                         norm2=NS(weight=rand(dim) * 0.1 + 1, eps=1e-5), residual_in_fp32=residual_in_fp32))
+            attn.conv1d = _Holder()
+            attn.conv1d.weight = torch.nn.Parameter(rand(qkv_dim, 1, d_conv, std=d_conv ** -0.5))
+            attn.conv1d.bias = None
+        mlp = _Holder()
+        mlp.fc1 = linear(2 * hidden, dim)
+        mlp.fc2 = linear(dim, hidden)
+        block = _Holder()
+        block.attn, block.mlp, block.norm, block.norm2 = attn, mlp, norm(), norm()
+        block.residual_in_fp32 = residual_in_fp32
+        blocks.append(block)
         a_cache = NS(norm_input=rand(batch, seq_len, dim, dt=res_dtype if layer else dtype),
+                     norm_output=rand(batch, seq_len, dim),
                      q_rope=rand(batch, n_heads, seq_len, head_dim), k_expanded=rand(batch, n_heads, seq_len, head_dim),
-                     v_expanded=rand(batch, n_heads, seq_len, head_dim))
-        m_cache = NS(norm_input=rand(batch, seq_len, dim, dt=res_dtype), fc1_output=rand(batch, seq_len, 2 * hidden))
+                     v_expanded=rand(batch, n_heads, seq_len, head_dim),
+                     out_proj_input=rand(batch, seq_len, n_heads * head_dim))
+        m_cache = NS(norm_input=rand(batch, seq_len, dim, dt=res_dtype), norm_output=rand(batch, seq_len, dim),
+                     fc1_output=rand(batch, seq_len, 2 * hidden), down_input=rand(batch, seq_len, hidden))
         caches.append(NS(layer_index=layer, attention=a_cache, mlp=m_cache))
-    backend = NS(backbone=NS(blocks=blocks))
+    backend = _Holder()
+    backend.backbone = _Holder()
+    backend.backbone.blocks = torch.nn.ModuleList(blocks)
     cache = NS(region_index=0, layer_range=(0, layers), layer_caches=caches,
                region_input=rand(batch, seq_len, dim))
     return backend, cache
@@ -205,6 +234,62 @@ def region_section(steps: int = 5) -> dict:
     return {"region_input_pullback_bf16_L2_D768_B8_T1024_P64": measure_region(iters=steps)}
 
 
+def measure_lbi_step(*, regions=6, layers_per_region=2, dim=768, n_heads=12, head_dim=64, hidden=3072, d_conv=4,
+                     batch=8, seq_len=1024, interface_width=64, dtype=torch.bfloat16, warmup=1, iters=3,
+                     device="cuda") -> dict:
+    """Device work of one LBI scan backward step at the end-to-end configuration (12 layers in 6
+    regions of 2, interface width 64): per region the state-Jacobian build (region input pullback
+    for 64 directions) and the parameter VJP, then the interface suffix scan (cotangent chain over
+    the 5 inner Jacobians).  The forward caches are synthetic and shared by the six regions
+    (same shapes); the interface's own small MLP pullbacks and the readout/canvas VJPs are not part
+    of this library and are left out."""
+    from .backends import HipTransformerLowering
+    from .hip.interface import suffix_scan_cotangents
+
+    backend, cache = synthetic_region(dim=dim, n_heads=n_heads, n_kv_heads=n_heads, head_dim=head_dim, hidden=hidden,
+                                      layers=layers_per_region, d_conv=d_conv, batch=batch, seq_len=seq_len,
+                                      dtype=dtype, device=device)
+    gen = torch.Generator(device="cpu").manual_seed(2)
+    basis = (torch.randn(batch, interface_width, 1, dim, generator=gen) / seq_len).expand(-1, -1, seq_len, -1).to(device)
+    cot = torch.randn(batch, seq_len, dim, generator=gen).to(device)
+    jts = (torch.eye(interface_width) + 0.05 * torch.randn(batch, regions - 1, interface_width, interface_width,
+                                                          generator=gen)).to(device)
+    g_state = torch.randn(batch, interface_width, generator=gen).to(device)
+    lowering = HipTransformerLowering()
+    parts = {}
+
+    def pullbacks():
+        for _ in range(regions):
+            lowering.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=basis)
+
+    def vjps():
+        for _ in range(regions):
+            lowering.parameter_vjp(backend=backend, cache=cache, output_cotangent=cot)
+
+    def scan():
+        suffix_scan_cotangents(jts, g_state)
+
+    def whole():
+        pullbacks()
+        scan()
+        vjps()
+
+    for name, fn in (("state_jacobian_pullbacks", pullbacks), ("parameter_vjps", vjps), ("interface_scan", scan),
+                     ("step", whole)):
+        median_ms, best_ms, mean_ms, peak = time_call(fn, warmup=warmup, iters=iters)
+        parts[name] = {"median_ms": median_ms, "best_ms": best_ms, "peak_memory_bytes": peak}
+    return {
+        "workload": f"LBI scan backward step, device work: {regions} regions x {layers_per_region} layers, d_model {dim}, "
+                    f"{n_heads} heads x {head_dim}, hidden {hidden}, interface width {interface_width}, B={batch} "
+                    f"T={seq_len}, {str(dtype).replace('torch.', '')}, synthetic caches",
+        **parts,
+    }
+
+
+def lbi_step_section(steps: int = 3) -> dict:
+    return {"lbi_backward_step_bf16_L12_D768_B8_T1024_d64": measure_lbi_step(iters=steps)}
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
     ap.add_argument("--shapes", nargs="*", default=["1,8,128,64,4"], help="B,H,T,Dh,P tuples")
@@ -217,7 +302,13 @@ def main(argv=None) -> int:
     ap.add_argument("--region", action="store_true",
                     help="time the region-level input pullback at the end-to-end configuration instead")
     ap.add_argument("--basis", type=int, default=64, help="cotangent directions of the --region run")
+    ap.add_argument("--lbi-step", action="store_true",
+                    help="time the device work of one LBI scan backward step at the end-to-end configuration")
     args = ap.parse_args(argv)
+    if args.lbi_step:
+        print(json.dumps(measure_lbi_step(dtype=getattr(torch, args.dtype), warmup=args.warmup, iters=args.iters)),
+              flush=True)
+        return 0
     if args.region:
         print(json.dumps(measure_region(basis=args.basis, dtype=getattr(torch, args.dtype), warmup=args.warmup,
                                         iters=args.iters)), flush=True)

@@ -155,33 +155,42 @@ __global__ __launch_bounds__(256) void rmsnorm_pullback_kernel(const TB* __restr
 // Gated MLP pullback.  fc1_output rows are [up | gate]; the forward computed
 // down_input = up * silu(gate) with silu(gate) rounded to the storage type.
 // ---------------------------------------------------------------------------------------
+// One workgroup per token (b, t): the activation row is read and its silu terms are formed once,
+// then applied to the P cotangent rows of that token.
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void gated_mlp_pullback_kernel(const T* __restrict__ g_down_input,
                                                                  const T* __restrict__ fc1_output,
-                                                                 T* __restrict__ g_fc1_output, long long n_units, int P,
-                                                                 int T_len, int hidden) {
-    const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (unit >= n_units) return;
-    const int per_row = hidden / VEC;
-    const long long row = unit / per_row;
-    const int j = (int)(unit - row * per_row) * VEC;
-    const long long bp = row / T_len;
-    const int t = (int)(row - bp * T_len);
-    const long long act_row = (bp / P) * T_len + t;
-    Pack<T, VEC> g, up, gate, o_up, o_gate;
-    g.load(g_down_input + row * hidden + j);
-    up.load(fc1_output + act_row * 2 * hidden + j);
-    gate.load(fc1_output + act_row * 2 * hidden + hidden + j);
+                                                                 T* __restrict__ g_fc1_output, int P, int T_len,
+                                                                 int hidden) {
+    const int b = blockIdx.x / T_len, t = blockIdx.x - b * T_len;
+    const T* act_row = fc1_output + (long long)blockIdx.x * 2 * hidden;
+    const long long row0 = (long long)b * P * T_len + t;  // cotangent row of direction 0
+    for (int j = threadIdx.x * VEC; j < hidden; j += blockDim.x * VEC) {
+        Pack<T, VEC> up, gate;
+        up.load(act_row + j);
+        gate.load(act_row + hidden + j);
+        float act[VEC], dact[VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        const float z = gate.v[i];
-        const float sig = 1.0f / (1.0f + __expf(-z));
-        const float act = round_via<T>(z * sig);
-        o_up.v[i] = g.v[i] * act;
-        o_gate.v[i] = round_via<T>(g.v[i] * up.v[i]) * (sig * (1.0f + z * (1.0f - sig)));
+        for (int i = 0; i < VEC; ++i) {
+            const float z = gate.v[i];
+            const float sig = 1.0f / (1.0f + __expf(-z));
+            act[i] = round_via<T>(z * sig);
+            dact[i] = sig * (1.0f + z * (1.0f - sig));
+        }
+#pragma unroll 4
+        for (int p = 0; p < P; ++p) {
+            const long long row = row0 + (long long)p * T_len;
+            Pack<T, VEC> g, o_up, o_gate;
+            g.load(g_down_input + row * hidden + j);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                o_up.v[i] = g.v[i] * act[i];
+                o_gate.v[i] = round_via<T>(g.v[i] * up.v[i]) * dact[i];
+            }
+            o_up.store(g_fc1_output + row * 2 * hidden + j);
+            o_gate.store(g_fc1_output + row * 2 * hidden + hidden + j);
+        }
     }
-    o_up.store(g_fc1_output + row * 2 * hidden + j);
-    o_gate.store(g_fc1_output + row * 2 * hidden + hidden + j);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -308,7 +317,7 @@ __global__ __launch_bounds__(256) void qkv_pullback_kernel(const T* __restrict__
 // ---------------------------------------------------------------------------------------
 // One thread: VEC channels x RUN consecutive positions, KMAX >= ksize taps held in registers
 // (taps past ksize are zero), input rows read once per RUN outputs.
-template <typename T, int VEC, int KMAX, int RUN>
+template <typename T, int VEC, int KMAX, int RUN, bool EXACT>
 __global__ __launch_bounds__(256) void causal_conv1d_pullback_kernel(const T* __restrict__ g_out,
                                                                      const T* __restrict__ weight, T* __restrict__ g_in,
                                                                      long long n_units, int T_len, int C, int ksize) {
@@ -322,11 +331,25 @@ __global__ __launch_bounds__(256) void causal_conv1d_pullback_kernel(const T* __
     const long long n = rest / n_runs;
 
     float tap[KMAX][VEC];  // tap[i][e] multiplies g_out at offset +i
+    if (EXACT) {
+        // ksize == KMAX: the VEC x KMAX weights of these channels are one contiguous, aligned span
+        Pack<T, VEC> wv[KMAX];
 #pragma unroll
-    for (int i = 0; i < KMAX; ++i)
+        for (int u = 0; u < KMAX; ++u) wv[u].load(weight + (long long)c0 * KMAX + u * VEC);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e)
-            tap[i][e] = i < ksize ? to_f32(weight[(long long)(c0 + e) * ksize + (ksize - 1 - i)]) : 0.0f;
+        for (int i = 0; i < KMAX; ++i)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const int flat = e * KMAX + (KMAX - 1 - i);
+                tap[i][e] = wv[flat / VEC].v[flat % VEC];
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < KMAX; ++i)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                tap[i][e] = i < ksize ? to_f32(weight[(long long)(c0 + e) * ksize + (ksize - 1 - i)]) : 0.0f;
+    }
     float acc[RUN][VEC];
 #pragma unroll
     for (int r = 0; r < RUN; ++r)
@@ -396,19 +419,20 @@ int launch_rmsnorm_x(int x_dtype, const void* g_out, const void* x, const void* 
 }
 
 template <typename T, int VEC>
-int launch_gated_as(const void* g, const void* fc1, void* out, long long n_rows, int P, int T_len, int hidden,
+int launch_gated_as(const void* g, const void* fc1, void* out, long long n_tokens, int P, int T_len, int hidden,
                     hipStream_t stream) {
-    const long long units = n_rows * (hidden / VEC);
-    if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many elements");
-    hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, VEC>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
-                       (const T*)g, (const T*)fc1, (T*)out, units, P, T_len, hidden);
+    if (n_tokens > 0x7fffffffLL) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many tokens");
+    const int chunks = hidden / VEC;
+    const int threads = chunks >= 256 ? 256 : ((chunks + 63) / 64) * 64;
+    hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, VEC>), dim3((unsigned)n_tokens), dim3(threads), 0, stream,
+                       (const T*)g, (const T*)fc1, (T*)out, P, T_len, hidden);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
 
 template <typename T>
 int launch_gated(const void* g, const void* fc1, void* out, long long n_rows, int P, int T_len, int hidden,
-                 hipStream_t stream) {
+                 hipStream_t stream) {  // n_rows: tokens B * T
     constexpr int W = wide<T>();
     const bool aligned =
         (reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(fc1) | reinterpret_cast<uintptr_t>(out)) % 16 == 0;
@@ -438,12 +462,12 @@ int launch_qkv(const void* dq, const void* dk, const void* dv, const float* cos_
     return LBI_OK;
 }
 
-template <typename T, int VEC, int KMAX, int RUN>
+template <typename T, int VEC, int KMAX, int RUN, bool EXACT = false>
 int launch_conv_as(const void* g_out, const void* weight, void* g_in, long long n_seq, int T_len, int C, int ksize,
                    hipStream_t stream) {
     const long long units = n_seq * ((T_len + RUN - 1) / RUN) * (C / VEC);
     if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_causal_conv1d_pullback: too many elements");
-    hipLaunchKernelGGL((causal_conv1d_pullback_kernel<T, VEC, KMAX, RUN>), dim3(blocks_for(units, 256)), dim3(256), 0,
+    hipLaunchKernelGGL((causal_conv1d_pullback_kernel<T, VEC, KMAX, RUN, EXACT>), dim3(blocks_for(units, 256)), dim3(256), 0,
                        stream, (const T*)g_out, (const T*)weight, (T*)g_in, units, T_len, C, ksize);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
@@ -455,7 +479,9 @@ int launch_conv(const void* g_out, const void* weight, void* g_in, long long n_s
     constexpr int W = wide<T>();
     const bool aligned = (reinterpret_cast<uintptr_t>(g_out) | reinterpret_cast<uintptr_t>(g_in)) % 16 == 0;
     if (C % W == 0 && aligned) {
-        if (ksize <= 4) return launch_conv_as<T, W, 4, 16>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
+        if (ksize == 4 && reinterpret_cast<uintptr_t>(weight) % 16 == 0)
+            return launch_conv_as<T, W, 4, 8, true>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
+        if (ksize <= 4) return launch_conv_as<T, W, 4, 8>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
         if (ksize <= 8) return launch_conv_as<T, W, 8, 8>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
     }
     if (ksize <= 4) return launch_conv_as<T, 1, 4, 8>(g_out, weight, g_in, n_seq, T_len, C, ksize, stream);
@@ -502,8 +528,8 @@ extern "C" int lbi_gated_mlp_pullback(const void* g_down_input, const void* fc1_
     if (!region::valid_dtype(dtype)) return fail(LBI_ERR_INVALID, "lbi_gated_mlp_pullback: bad dtype %d", dtype);
     if (B < 0 || P < 0 || T < 0 || !region::positive_int(hidden) || P > 0x7fffffff || T > 0x7fffffff)
         return fail(LBI_ERR_INVALID, "lbi_gated_mlp_pullback: bad size");
-    const long long n_rows = (long long)B * P * T;
-    if (n_rows == 0) return LBI_OK;
+    if (B == 0 || P == 0 || T == 0) return LBI_OK;
+    const long long n_rows = (long long)B * T;  // one workgroup per token
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case LBI_F32: return region::launch_gated<float>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, s);
