@@ -157,6 +157,13 @@ def causal_conv1d_pullback(g_out: torch.Tensor, weight: torch.Tensor) -> torch.T
     return out
 
 
+def _apply_transposed(g: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``g @ weight`` for ``weight [out, in]``: the pullback of ``y = x weight^T``.  Issued as
+    the library's ``A B^T`` form on a transposed copy of the (small) weight, which is its faster
+    path for these tall products."""
+    return torch.nn.functional.linear(g, weight.t().contiguous())
+
+
 def _rows(t: torch.Tensor) -> torch.Tensor:
     return t.reshape(-1, t.shape[-1])
 
@@ -219,12 +226,12 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
     # gated MLP: hidden_out = fc2(up * silu(gate)), [up | gate] = fc1(norm2(res2))
     if param_grads is not None:
         _linear_grads(param_grads, mlp.fc2, g_hidden, m_cache.down_input)
-    g_down_input = torch.matmul(g_hidden, mlp.fc2.weight)
+    g_down_input = _apply_transposed(g_hidden, mlp.fc2.weight)
     g_fc1 = gated_mlp_pullback(g_down_input, m_cache.fc1_output)
     del g_down_input
     if param_grads is not None:
         _linear_grads(param_grads, mlp.fc1, g_fc1, m_cache.norm_output)
-    g_norm2 = torch.matmul(g_fc1, mlp.fc1.weight)
+    g_norm2 = _apply_transposed(g_fc1, mlp.fc1.weight)
     del g_fc1
     if param_grads is not None:
         _norm_weight_grad(param_grads, block.norm2, g_norm2, m_cache.norm_input)
@@ -236,7 +243,7 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
     # attention: res2 = out_proj(heads) + res1
     if param_grads is not None:
         _linear_grads(param_grads, attn.out_proj, g_attn_out, a_cache.out_proj_input)
-    g_merged = torch.matmul(g_attn_out, attn.out_proj.weight)
+    g_merged = _apply_transposed(g_attn_out, attn.out_proj.weight)
     del g_attn_out
     g_heads = attn_heads_split(g_merged, attn.n_heads, attn.head_dim)
     del g_merged
@@ -257,7 +264,7 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
         g_qkv = causal_conv1d_pullback(g_qkv, attn.conv1d.weight)
     if param_grads is not None:
         _linear_grads(param_grads, attn.in_proj, g_qkv, a_cache.norm_output)
-    g_norm1 = torch.matmul(g_qkv, attn.in_proj.weight)
+    g_norm1 = _apply_transposed(g_qkv, attn.in_proj.weight)
     del g_qkv
     if param_grads is not None:
         _norm_weight_grad(param_grads, block.norm, g_norm1, a_cache.norm_input)
