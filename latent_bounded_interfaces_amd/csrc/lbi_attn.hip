@@ -3,6 +3,7 @@
 #include "lbi_attn_generic.h"
 #include "lbi_attn_mfma.h"
 #include "lbi_attn_dkdv128.h"
+#include "lbi_attn_dkdv_pair.h"
 #include "lbi_attn_dq128.h"
 
 namespace lbi {

@@ -362,6 +362,11 @@ template <typename T, int DH, bool CAUSAL>
 void launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
                  int n_bh, int H, int P, int T_len, float scale, hipStream_t stream);
 
+// dK/dV launch for two or more directions (kernel in lbi_attn_dkdv_pair.h).
+template <typename T, int DH, bool CAUSAL>
+void launch_dkdv_pair(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk,
+                      T* dv, int n_bh, int H, int P, int T_len, float scale, hipStream_t stream);
+
 // dQ launch (kernel in lbi_attn_dq128.h); PB = directions per wave.
 template <typename T, int DH, int PB, bool CAUSAL>
 void launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
@@ -384,7 +389,8 @@ int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T
                        dim3(256), 0, stream, g, o32, delta, H, P, T_len, n_rows);
     if (DH == 64 && P > 4) launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
     else launch_dq<T, DH, 4, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
+    if (P >= 2) launch_dkdv_pair<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
+    else launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
