@@ -78,13 +78,17 @@ __global__ __launch_bounds__(256) void dkdv_pair_kernel(const T* __restrict__ q,
 
     // ---- global -> LDS.  The 3 CPT wave-loads of a stage are dealt round-robin: wave w takes
     // loads w, w + 4, ...; load c belongs to tile c / CPT and is its wave-load u = c % CPT.
-    unsigned dma_off[NXW];
+    unsigned dma_off[NXW], dma_dst[NXW];   // lane offset inside the source tile; LDS offset inside a stage
+    const T* dma_src[NXW];                 // wave-uniform source of each wave-load
 #pragma unroll
     for (int x = 0; x < NXW; ++x) {
-        const int u = (wave + 4 * x) % CPT;
+        const int c = wave + 4 * x;
+        const int tile = c / CPT, u = c % CPT;
         const int sigma = 64 * u + lane;
         const int r = sigma / CPR;
         dma_off[x] = r * RB + (((sigma % CPR) ^ swz<DH>(r)) << 4);
+        dma_dst[x] = tile * TILE + 1024 * u;
+        dma_src[x] = tile == 0 ? q_bh : d_out + prow[tile - 1] * DH;
     }
     // lanes 0-7: lse2, 8-15: -delta of direction 0, 16-23: of direction 1 (float4 each)
     const float* stat_ptr = (lane < 8 ? lse_bh : delta + prow[lane < 16 ? 0 : 1]) + 4 * (lane & 7);
@@ -92,12 +96,7 @@ __global__ __launch_bounds__(256) void dkdv_pair_kernel(const T* __restrict__ q,
     auto issue_tile = [&](int i_row, unsigned stage_base) __attribute__((always_inline)) {
         const unsigned row_bytes = (unsigned)i_row * RB;
 #pragma unroll
-        for (int x = 0; x < NXW; ++x) {
-            const int c = wave + 4 * x;              // wave-uniform
-            const int tile = c / CPT, u = c % CPT;
-            const T* src = tile == 0 ? q_bh : d_out + prow[tile - 1] * DH;
-            dma16(src, row_bytes + dma_off[x], lds0 + stage_base + tile * TILE + 1024 * u);
-        }
+        for (int x = 0; x < NXW; ++x) dma16(dma_src[x], row_bytes + dma_off[x], lds0 + stage_base + dma_dst[x]);
         if (lane < 24) dma16_at(stat_ptr + i_row, lds0 + stage_base + 3 * TILE + 512 * wave);
     };
 
