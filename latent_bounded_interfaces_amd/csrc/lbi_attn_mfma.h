@@ -319,33 +319,40 @@ __global__ __launch_bounds__(256) void stats_kernel(const T* __restrict__ q, con
 }
 
 // ---------------------------------------------------------------------------------------
-// delta_kernel: DH/8 lanes per row, 16 bytes of d_out and 32 bytes of O per lane.
+// delta_kernel: DH/8 lanes per (b, h, t) row; a lane keeps its 32 bytes of O and walks the P
+// directions (16 bytes of d_out each), so O is read once and no index is divided per element.
 // ---------------------------------------------------------------------------------------
 template <typename T, int DH>
 __global__ __launch_bounds__(256) void delta_kernel(const T* __restrict__ d_out, const float* __restrict__ o32,
-                                                    float* __restrict__ delta, int H, int P, int T_len,
-                                                    size_t n_rows) {
-    constexpr int LPR = DH / 8;  // lanes per row
-    const size_t row = (size_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
+                                                    float* __restrict__ delta, int H, int P, int T_len) {
+    constexpr int LPR = DH / 8;           // lanes per row
+    constexpr int ROWS = 256 / LPR;       // rows per workgroup
+    const int n_chunks = (T_len + ROWS - 1) / ROWS;
+    const int bh = blockIdx.x / n_chunks;  // b * H + h
+    const int t = (blockIdx.x - bh * n_chunks) * ROWS + threadIdx.x / LPR;
     const int part = threadIdx.x % LPR;
-    float acc = 0.0f;
-    if (row < n_rows) {
-        const size_t t = row % T_len;
-        const size_t bph = row / T_len;
-        const size_t h = bph % H, b = bph / ((size_t)H * P);
-        const size_t o_row = (b * H + h) * T_len + t;
+    const bool valid = t < T_len;
+    const int tc = valid ? t : T_len - 1;
+    const int b = bh / H, h = bh - b * H;
+    const float* o_ptr = o32 + ((size_t)bh * T_len + tc) * DH + part * 8;
+    const f32x4 o_lo = *reinterpret_cast<const f32x4*>(o_ptr);
+    const f32x4 o_hi = *reinterpret_cast<const f32x4*>(o_ptr + 4);
+    const size_t row0 = ((size_t)b * P * H + h) * T_len + tc;   // direction 0; + p * H * T_len
+    const size_t p_stride = (size_t)H * T_len;
+#pragma unroll 4
+    for (int p = 0; p < P; ++p) {
+        const size_t row = row0 + p * p_stride;
         const u32x4 g = *reinterpret_cast<const u32x4*>(d_out + row * DH + part * 8);
-        const f32x4 o_lo = *reinterpret_cast<const f32x4*>(o32 + o_row * DH + part * 8);
-        const f32x4 o_hi = *reinterpret_cast<const f32x4*>(o32 + o_row * DH + part * 8 + 4);
         const T* ge = reinterpret_cast<const T*>(&g);
+        float acc = 0.0f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc = fmaf(to_f32(ge[e]), o_lo[e], acc);
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc = fmaf(to_f32(ge[4 + e]), o_hi[e], acc);
-    }
 #pragma unroll
-    for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, LPR);
-    if (part == 0 && row < n_rows) delta[row] = -acc;  // stored negated: the dK/dV kernel starts dP from it
+        for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, LPR);
+        if (part == 0 && valid) delta[row] = -acc;  // stored negated: the dK/dV kernel starts dP from it
+    }
 }
 
 inline bool supports(int T_len, int dh, int dtype) {
@@ -383,10 +390,9 @@ int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T
     const int n_qb = (T_len + 127) / 128;
     hipLaunchKernelGGL((stats_kernel<T, DH, CAUSAL>), dim3(grid_size(n_qb, n_bh)), dim3(256), lds_bytes, stream, q, k,
                        v, lse2, o32, n_bh, T_len, scale);
-    const size_t n_rows = (size_t)n_bh * P * T_len;
     constexpr int rows_per_block = 256 / (DH / 8);
-    hipLaunchKernelGGL((delta_kernel<T, DH>), dim3((unsigned)((n_rows + rows_per_block - 1) / rows_per_block)),
-                       dim3(256), 0, stream, g, o32, delta, H, P, T_len, n_rows);
+    hipLaunchKernelGGL((delta_kernel<T, DH>), dim3((unsigned)((T_len + rows_per_block - 1) / rows_per_block) * n_bh),
+                       dim3(256), 0, stream, g, o32, delta, H, P, T_len);
     if (DH == 64 && P > 4) launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
     else launch_dq<T, DH, 4, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
     if (P >= 2) launch_dkdv_pair<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
