@@ -192,6 +192,22 @@ int lbi_attn_qkv_pullback(const void* dq, const void* dk, const void* dv,
 int lbi_causal_conv1d_pullback(const void* g_out, const void* weight, void* g_in,
                                int64_t N, int64_t T, int64_t C, int64_t ksize, int dtype, void* stream);
 
+/*
+ * lbi_attn_qkv_pullback followed by lbi_causal_conv1d_pullback in one pass, without storing the
+ * cotangent of the convolved projection (reference backends/transformer.py:121-132 transposed):
+ *
+ *   dq, dk, dv [B,P,H,T,Dh], conv_weight [(H + 2*Hkv)*Dh, k]  ->  g_in [B,P,T,(H + 2*Hkv)*Dh]
+ *
+ * The intermediate is rounded to the storage type as the two calls would store it and the sums run
+ * in the same order: fp32 results are bit-identical to theirs, 16-bit results equal up to the last
+ * place of a final rounding.  k <= 8; longer filters return LBI_ERR_UNSUPPORTED and take the two
+ * calls.
+ */
+int lbi_attn_qkv_conv_pullback(const void* dq, const void* dk, const void* dv,
+                               const float* rope_cos, const float* rope_sin, const void* conv_weight,
+                               void* g_in, int64_t B, int64_t P, int64_t T, int64_t H, int64_t Hkv,
+                               int64_t Dh, int interleaved, int64_t ksize, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

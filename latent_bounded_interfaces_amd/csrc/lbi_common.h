@@ -41,12 +41,9 @@ __device__ __forceinline__ float to_f32(float x) { return x; }
 __device__ __forceinline__ float to_f32(_Float16 x) { return (float)x; }
 __device__ __forceinline__ float to_f32(bf16_raw x) { return __uint_as_float(((unsigned)x.bits) << 16); }
 
-// Round-to-nearest-even narrowing, NaN preserved as quiet NaN.
+// Round-to-nearest-even narrowing (NaN stays a quiet NaN): the hardware conversion, v_cvt_pk_bf16_f32.
 __device__ __forceinline__ unsigned short f32_to_bf16_bits(float x) {
-    unsigned u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (unsigned short)(u >> 16);
+    return __builtin_bit_cast(unsigned short, (__bf16)x);
 }
 
 // Four consecutive storage elements widened to fp32 with one vector load.

@@ -217,31 +217,25 @@ __global__ __launch_bounds__(256) void heads_split_kernel(const CHUNK* __restric
 // (j, j + Dh/2) or, interleaved, (2j, 2j + 1); R^T: (ge cos + go sin, -ge sin + go cos).
 // One thread handles VEC pairs of one rotary head, or 2 VEC value elements.
 // ---------------------------------------------------------------------------------------
-template <typename T, int VEC>
-__global__ __launch_bounds__(256) void qkv_pullback_kernel(const T* __restrict__ dq, const T* __restrict__ dk,
-                                                           const T* __restrict__ dv, const float* __restrict__ cos_t,
-                                                           const float* __restrict__ sin_t, T* __restrict__ out,
-                                                           long long n_units, int T_len, int H, int Hkv, int Dh,
-                                                           int interleaved) {
-    const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (unit >= n_units) return;
+// Cotangent of the packed projection for one (n, t), one packed head and VEC rotary pairs starting at pair j
+// (or 2 VEC value elements): sums the query heads of a key/value group, applies the transposed rotation.
+// y0 / y1 are the values at in-head offsets off0.. / off1.. (see qkv_unit_offsets).
+template <int VEC, bool INTERLEAVED>
+__device__ __forceinline__ void qkv_unit_offsets(bool rotary, int half, int j, int& off0, int& off1) {
+    off0 = (rotary && !INTERLEAVED) ? j : 2 * j;
+    off1 = (rotary && !INTERLEAVED) ? half + j : 2 * j + VEC;
+}
+
+template <typename T, int VEC, bool INTERLEAVED>
+__device__ __forceinline__ void qkv_unit_values(const T* __restrict__ dq, const T* __restrict__ dk,
+                                                const T* __restrict__ dv, const float* __restrict__ cos_t,
+                                                const float* __restrict__ sin_t, long long n, int t, int T_len, int H,
+                                                int Hkv, int Dh, int head, int j, float (&y0)[VEC], float (&y1)[VEC]) {
     const int half = Dh / 2;
-    const int upr = half / VEC;                  // units per head (rotary pair groups, or 2 VEC value elements)
-    const int per_token = (H + 2 * Hkv) * upr;
-    const long long row = unit / per_token;      // (n, t)
-    const int u = (int)(unit - row * per_token);
-    const int head = u / upr;                    // packed head index: q heads, then k heads, then v heads
-    const int j = (u - head * upr) * VEC;
-    const long long n = row / T_len;
-    const int t = (int)(row - n * T_len);
     const int rep = H / Hkv;
-    T* o_row = out + row * (long long)(H + 2 * Hkv) * Dh + (long long)head * Dh;
-
-    // first / second storage offsets of this unit inside a head
     const bool rotary = head < H + Hkv;
-    const int off0 = (rotary && !interleaved) ? j : 2 * j;
-    const int off1 = (rotary && !interleaved) ? half + j : 2 * j + VEC;
-
+    int off0, off1;
+    qkv_unit_offsets<VEC, INTERLEAVED>(rotary, half, j, off0, off1);
     const T* src;
     int first_head, count;
     if (head < H) {
@@ -265,49 +259,179 @@ __global__ __launch_bounds__(256) void qkv_pullback_kernel(const T* __restrict__
             a1[i] += x1.v[i];
         }
     }
-    Pack<T, VEC> y0, y1;
     if (!rotary) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-            y0.v[i] = a0[i];
-            y1.v[i] = a1[i];
+            y0[i] = a0[i];
+            y1[i] = a1[i];
         }
-    } else {
-        Pack<float, VEC> cs, sn;
-        cs.load(cos_t + (long long)t * half + j);
-        sn.load(sin_t + (long long)t * half + j);
-        float ge[VEC], go[VEC];
+        return;
+    }
+    Pack<float, VEC> cs, sn;
+    cs.load(cos_t + (long long)t * half + j);
+    sn.load(sin_t + (long long)t * half + j);
+    float ge[VEC], go[VEC];
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            if (interleaved) {  // a0|a1 holds pairs (2i, 2i+1) of the 2 VEC span
-                const int e = 2 * i, o = 2 * i + 1;
-                ge[i] = e < VEC ? a0[e % VEC] : a1[e % VEC];
-                go[i] = o < VEC ? a0[o % VEC] : a1[o % VEC];
-            } else {
-                ge[i] = a0[i];
-                go[i] = a1[i];
-            }
+    for (int i = 0; i < VEC; ++i) {
+        if (INTERLEAVED) {  // a0|a1 holds pairs (2i, 2i+1) of the 2 VEC span
+            const int e = 2 * i, o = 2 * i + 1;
+            ge[i] = e < VEC ? a0[e % VEC] : a1[e % VEC];
+            go[i] = o < VEC ? a0[o % VEC] : a1[o % VEC];
+        } else {
+            ge[i] = a0[i];
+            go[i] = a1[i];
         }
-        float re[VEC], ro[VEC];
+    }
+    float re[VEC], ro[VEC];
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            re[i] = ge[i] * cs.v[i] + go[i] * sn.v[i];
-            ro[i] = go[i] * cs.v[i] - ge[i] * sn.v[i];
-        }
+    for (int i = 0; i < VEC; ++i) {
+        // explicit fused steps: every caller rounds the same way whatever the compiler would contract
+        re[i] = fmaf(ge[i], cs.v[i], go[i] * sn.v[i]);
+        ro[i] = fmaf(go[i], cs.v[i], -(ge[i] * sn.v[i]));
+    }
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            if (interleaved) {
-                const int e = 2 * i, o = 2 * i + 1;
-                if (e < VEC) y0.v[e % VEC] = re[i]; else y1.v[e % VEC] = re[i];
-                if (o < VEC) y0.v[o % VEC] = ro[i]; else y1.v[o % VEC] = ro[i];
-            } else {
-                y0.v[i] = re[i];
-                y1.v[i] = ro[i];
-            }
+    for (int i = 0; i < VEC; ++i) {
+        if (INTERLEAVED) {
+            const int e = 2 * i, o = 2 * i + 1;
+            if (e < VEC) y0[e % VEC] = re[i]; else y1[e % VEC] = re[i];
+            if (o < VEC) y0[o % VEC] = ro[i]; else y1[o % VEC] = ro[i];
+        } else {
+            y0[i] = re[i];
+            y1[i] = ro[i];
         }
+    }
+}
+
+template <typename T, int VEC, bool INTERLEAVED>
+__global__ __launch_bounds__(256) void qkv_pullback_kernel(const T* __restrict__ dq, const T* __restrict__ dk,
+                                                           const T* __restrict__ dv, const float* __restrict__ cos_t,
+                                                           const float* __restrict__ sin_t, T* __restrict__ out,
+                                                           long long n_units, int T_len, int H, int Hkv, int Dh) {
+    const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (unit >= n_units) return;
+    const int half = Dh / 2;
+    const int upr = half / VEC;                  // units per head (rotary pair groups, or 2 VEC value elements)
+    const int per_token = (H + 2 * Hkv) * upr;
+    const long long row = unit / per_token;      // (n, t)
+    const int u = (int)(unit - row * per_token);
+    const int head = u / upr;                    // packed head index: q heads, then k heads, then v heads
+    const int j = (u - head * upr) * VEC;
+    const long long n = row / T_len;
+    const int t = (int)(row - n * T_len);
+    T* o_row = out + row * (long long)(H + 2 * Hkv) * Dh + (long long)head * Dh;
+    int off0, off1;
+    qkv_unit_offsets<VEC, INTERLEAVED>(head < H + Hkv, half, j, off0, off1);
+    float v0[VEC], v1[VEC];
+    qkv_unit_values<T, VEC, INTERLEAVED>(dq, dk, dv, cos_t, sin_t, n, t, T_len, H, Hkv, Dh, head, j, v0, v1);
+    Pack<T, VEC> y0, y1;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        y0.v[i] = v0[i];
+        y1.v[i] = v1[i];
     }
     y0.store(o_row + off0);
     y1.store(o_row + off1);
+}
+
+// The same projection cotangent pulled back through the depthwise causal convolution that follows the packed
+// projection (see the transposed convolution below), without storing the intermediate: one thread forms the
+// projection cotangent of its 2 VEC channels at RUN + KMAX - 1 consecutive positions and accumulates RUN outputs.
+template <typename T, int VEC, int KMAX, int RUN, bool INTERLEAVED, bool EXACT>
+__global__ __launch_bounds__(256) void qkv_conv_pullback_kernel(const T* __restrict__ dq, const T* __restrict__ dk,
+                                                                const T* __restrict__ dv,
+                                                                const float* __restrict__ cos_t,
+                                                                const float* __restrict__ sin_t,
+                                                                const T* __restrict__ weight, T* __restrict__ out,
+                                                                long long n_units, int T_len, int H, int Hkv, int Dh,
+                                                                int ksize) {
+    const long long unit = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (unit >= n_units) return;
+    const int half = Dh / 2;
+    const int upr = half / VEC;
+    const int per_token = (H + 2 * Hkv) * upr;
+    const int n_runs = (T_len + RUN - 1) / RUN;
+    const int u = (int)(unit % per_token);
+    const long long rest = unit / per_token;
+    const int s0 = (int)(rest % n_runs) * RUN;
+    const long long n = rest / n_runs;
+    const int head = u / upr;
+    const int j = (u - head * upr) * VEC;
+    const int C = (H + 2 * Hkv) * Dh;
+    int off0, off1;
+    qkv_unit_offsets<VEC, INTERLEAVED>(head < H + Hkv, half, j, off0, off1);
+    const int c0 = head * Dh + off0, c1 = head * Dh + off1;
+
+    float tap0[KMAX][VEC], tap1[KMAX][VEC];  // tap[i][e] multiplies the projection cotangent at offset +i
+    if (EXACT) {
+        // ksize == KMAX: the VEC x KMAX weights of a channel group are one contiguous, aligned span
+        Pack<T, VEC> w0[KMAX], w1[KMAX];
+#pragma unroll
+        for (int u2 = 0; u2 < KMAX; ++u2) {
+            w0[u2].load(weight + (long long)c0 * KMAX + u2 * VEC);
+            w1[u2].load(weight + (long long)c1 * KMAX + u2 * VEC);
+        }
+#pragma unroll
+        for (int i = 0; i < KMAX; ++i)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const int flat = e * KMAX + (KMAX - 1 - i);
+                tap0[i][e] = w0[flat / VEC].v[flat % VEC];
+                tap1[i][e] = w1[flat / VEC].v[flat % VEC];
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < KMAX; ++i)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                tap0[i][e] = i < ksize ? to_f32(weight[(long long)(c0 + e) * ksize + (ksize - 1 - i)]) : 0.0f;
+                tap1[i][e] = i < ksize ? to_f32(weight[(long long)(c1 + e) * ksize + (ksize - 1 - i)]) : 0.0f;
+            }
+    }
+    float acc0[RUN][VEC], acc1[RUN][VEC];
+#pragma unroll
+    for (int r = 0; r < RUN; ++r)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc0[r][e] = acc1[r][e] = 0.0f;
+    T* o = out + (n * T_len + s0) * (long long)C;
+#pragma unroll
+    for (int jj = 0; jj < RUN + KMAX - 1; ++jj) {
+        float g0[VEC], g1[VEC];
+        if (s0 + jj < T_len && jj < RUN + ksize - 1) {
+            qkv_unit_values<T, VEC, INTERLEAVED>(dq, dk, dv, cos_t, sin_t, n, s0 + jj, T_len, H, Hkv, Dh, head, j, g0,
+                                                 g1);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {  // the stored intermediate of the two-kernel form is rounded to T
+                g0[e] = round_via<T>(g0[e]);
+                g1[e] = round_via<T>(g1[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) g0[e] = g1[e] = 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < RUN; ++r) {
+            const int i = jj - r;
+            if (i >= 0 && i < KMAX) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    acc0[r][e] = fmaf(tap0[i][e], g0[e], acc0[r][e]);
+                    acc1[r][e] = fmaf(tap1[i][e], g1[e], acc1[r][e]);
+                }
+            }
+        }
+        // output jj - (KMAX - 1) has now seen its last row: store it, so only KMAX outputs are live at a time
+        const int r = jj - (KMAX - 1);
+        if (r >= 0 && r < RUN && s0 + r < T_len) {
+            Pack<T, VEC> y0, y1;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                y0.v[e] = acc0[r][e];
+                y1.v[e] = acc1[r][e];
+            }
+            y0.store(o + (long long)r * C + c0);
+            y1.store(o + (long long)r * C + c1);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -445,21 +569,62 @@ template <typename T>
 int launch_qkv(const void* dq, const void* dk, const void* dv, const float* cos_t, const float* sin_t, void* out,
                long long n_rows, int T_len, int H, int Hkv, int Dh, int interleaved, hipStream_t stream) {
     const int half = Dh / 2;
-    if (half % 4 == 0) {
-        const long long units = n_rows * (long long)(H + 2 * Hkv) * (half / 4);
-        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_qkv_pullback: too many elements");
-        hipLaunchKernelGGL((qkv_pullback_kernel<T, 4>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
-                           (const T*)dq, (const T*)dk, (const T*)dv, cos_t, sin_t, (T*)out, units, T_len, H, Hkv, Dh,
-                           interleaved);
+    const int vec = half % 4 == 0 ? 4 : 1;
+    const long long units = n_rows * (long long)(H + 2 * Hkv) * (half / vec);
+    if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_qkv_pullback: too many elements");
+    const dim3 grid(blocks_for(units, 256)), block(256);
+#define LBI_QKV_LAUNCH(VEC, IL)                                                                                       \
+    hipLaunchKernelGGL((qkv_pullback_kernel<T, VEC, IL>), grid, block, 0, stream, (const T*)dq, (const T*)dk,        \
+                       (const T*)dv, cos_t, sin_t, (T*)out, units, T_len, H, Hkv, Dh)
+    if (vec == 4) {
+        if (interleaved) LBI_QKV_LAUNCH(4, true); else LBI_QKV_LAUNCH(4, false);
     } else {
-        const long long units = n_rows * (long long)(H + 2 * Hkv) * half;
-        if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_qkv_pullback: too many elements");
-        hipLaunchKernelGGL((qkv_pullback_kernel<T, 1>), dim3(blocks_for(units, 256)), dim3(256), 0, stream,
-                           (const T*)dq, (const T*)dk, (const T*)dv, cos_t, sin_t, (T*)out, units, T_len, H, Hkv, Dh,
-                           interleaved);
+        if (interleaved) LBI_QKV_LAUNCH(1, true); else LBI_QKV_LAUNCH(1, false);
     }
+#undef LBI_QKV_LAUNCH
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
+}
+
+template <typename T, int VEC, int KMAX, bool INTERLEAVED, bool EXACT>
+int launch_qkv_conv_as(const void* dq, const void* dk, const void* dv, const float* cos_t, const float* sin_t,
+                       const void* weight, void* out, long long n_seq, int T_len, int H, int Hkv, int Dh, int ksize,
+                       hipStream_t stream) {
+    constexpr int RUN = KMAX <= 4 ? 16 : 8;  // longer runs spill
+    const long long units = n_seq * ((T_len + RUN - 1) / RUN) * (long long)(H + 2 * Hkv) * (Dh / 2 / VEC);
+    if (!fits_grid(units, 256)) return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_qkv_conv_pullback: too many elements");
+    hipLaunchKernelGGL((qkv_conv_pullback_kernel<T, VEC, KMAX, RUN, INTERLEAVED, EXACT>), dim3(blocks_for(units, 256)),
+                       dim3(256), 0, stream, (const T*)dq, (const T*)dk, (const T*)dv, cos_t, sin_t, (const T*)weight,
+                       (T*)out, units, T_len, H, Hkv, Dh, ksize);
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
+}
+
+template <typename T, bool INTERLEAVED>
+int launch_qkv_conv_il(const void* dq, const void* dk, const void* dv, const float* cos_t, const float* sin_t,
+                       const void* weight, void* out, long long n_seq, int T_len, int H, int Hkv, int Dh, int ksize,
+                       hipStream_t stream) {
+    const bool vec = (Dh / 2) % 4 == 0;
+    // the 4 x 4 weights of a channel group are contiguous; 4-element loads of them need 4-element alignment
+    const bool exact = vec && ksize == 4 && reinterpret_cast<uintptr_t>(weight) % (4 * sizeof(T)) == 0;
+    if (exact)
+        return launch_qkv_conv_as<T, 4, 4, INTERLEAVED, true>(dq, dk, dv, cos_t, sin_t, weight, out, n_seq, T_len, H, Hkv, Dh, ksize, stream);
+    if (vec && ksize <= 4)
+        return launch_qkv_conv_as<T, 4, 4, INTERLEAVED, false>(dq, dk, dv, cos_t, sin_t, weight, out, n_seq, T_len, H, Hkv, Dh, ksize, stream);
+    if (vec)
+        return launch_qkv_conv_as<T, 4, 8, INTERLEAVED, false>(dq, dk, dv, cos_t, sin_t, weight, out, n_seq, T_len, H, Hkv, Dh, ksize, stream);
+    if (ksize <= 4)
+        return launch_qkv_conv_as<T, 1, 4, INTERLEAVED, false>(dq, dk, dv, cos_t, sin_t, weight, out, n_seq, T_len, H, Hkv, Dh, ksize, stream);
+    return launch_qkv_conv_as<T, 1, 8, INTERLEAVED, false>(dq, dk, dv, cos_t, sin_t, weight, out, n_seq, T_len, H, Hkv, Dh, ksize, stream);
+}
+
+template <typename T>
+int launch_qkv_conv(const void* dq, const void* dk, const void* dv, const float* cos_t, const float* sin_t,
+                    const void* weight, void* out, long long n_seq, int T_len, int H, int Hkv, int Dh, int interleaved,
+                    int ksize, hipStream_t stream) {
+    if (interleaved)
+        return launch_qkv_conv_il<T, true>(dq, dk, dv, cos_t, sin_t, weight, out, n_seq, T_len, H, Hkv, Dh, ksize, stream);
+    return launch_qkv_conv_il<T, false>(dq, dk, dv, cos_t, sin_t, weight, out, n_seq, T_len, H, Hkv, Dh, ksize, stream);
 }
 
 template <typename T, int VEC, int KMAX, int RUN, bool EXACT = false>
@@ -592,6 +757,32 @@ extern "C" int lbi_attn_qkv_pullback(const void* dq, const void* dk, const void*
         case LBI_F32: return region::launch_qkv<float>(dq, dk, dv, rope_cos, rope_sin, g_qkv, n_rows, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, s);
         case LBI_F16: return region::launch_qkv<_Float16>(dq, dk, dv, rope_cos, rope_sin, g_qkv, n_rows, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, s);
         default: return region::launch_qkv<bf16_raw>(dq, dk, dv, rope_cos, rope_sin, g_qkv, n_rows, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, s);
+    }
+}
+
+extern "C" int lbi_attn_qkv_conv_pullback(const void* dq, const void* dk, const void* dv, const float* rope_cos,
+                                          const float* rope_sin, const void* conv_weight, void* g_in, int64_t B,
+                                          int64_t P, int64_t T, int64_t H, int64_t Hkv, int64_t Dh, int interleaved,
+                                          int64_t ksize, int dtype, void* stream) {
+    clear_error();
+    if (!dq || !dk || !dv || !rope_cos || !rope_sin || !conv_weight || !g_in)
+        return fail(LBI_ERR_INVALID, "lbi_attn_qkv_conv_pullback: null pointer");
+    if (!region::valid_dtype(dtype)) return fail(LBI_ERR_INVALID, "lbi_attn_qkv_conv_pullback: bad dtype %d", dtype);
+    if (B < 0 || P < 0 || !region::positive_int(T) || !region::positive_int(H) || !region::positive_int(Hkv) ||
+        !region::positive_int(Dh) || (long long)(H + 2 * Hkv) * Dh > 0x7fffffffLL)
+        return fail(LBI_ERR_INVALID, "lbi_attn_qkv_conv_pullback: bad size");
+    if (H % Hkv != 0) return fail(LBI_ERR_INVALID, "lbi_attn_qkv_conv_pullback: H=%lld not a multiple of Hkv=%lld", (long long)H, (long long)Hkv);
+    if (Dh % 2 != 0) return fail(LBI_ERR_INVALID, "lbi_attn_qkv_conv_pullback: rotary embedding needs an even head dim, got %lld", (long long)Dh);
+    if (ksize < 1) return fail(LBI_ERR_INVALID, "lbi_attn_qkv_conv_pullback: bad filter length %lld", (long long)ksize);
+    if (ksize > 8)
+        return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_qkv_conv_pullback: filter length %lld above 8; call lbi_attn_qkv_pullback and lbi_causal_conv1d_pullback", (long long)ksize);
+    const long long n_seq = (long long)B * P;
+    if (n_seq == 0) return LBI_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case LBI_F32: return region::launch_qkv_conv<float>(dq, dk, dv, rope_cos, rope_sin, conv_weight, g_in, n_seq, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, (int)ksize, s);
+        case LBI_F16: return region::launch_qkv_conv<_Float16>(dq, dk, dv, rope_cos, rope_sin, conv_weight, g_in, n_seq, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, (int)ksize, s);
+        default: return region::launch_qkv_conv<bf16_raw>(dq, dk, dv, rope_cos, rope_sin, conv_weight, g_in, n_seq, (int)T, (int)H, (int)Hkv, (int)Dh, interleaved != 0, (int)ksize, s);
     }
 }
 

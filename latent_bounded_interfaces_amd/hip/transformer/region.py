@@ -157,6 +157,38 @@ def causal_conv1d_pullback(g_out: torch.Tensor, weight: torch.Tensor) -> torch.T
     return out
 
 
+#: longest convolution filter the one-pass projection + convolution pullback takes
+FUSED_CONV_MAX_TAPS = 8
+
+
+def attn_qkv_conv_pullback(dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor, conv_weight: torch.Tensor, *,
+                           n_kv_heads: int, rope_base: float, rope_interleaved: bool) -> torch.Tensor:
+    """:func:`attn_qkv_pullback` then :func:`causal_conv1d_pullback` in one pass over ``dq, dk, dv``
+    (same arithmetic as the two calls, bit-identical in fp32; filters of at most ``FUSED_CONV_MAX_TAPS`` taps)."""
+    _require_cuda(dq, dk, dv, conv_weight)
+    bsz, basis, heads, seqlen, head_dim = dq.shape
+    if dk.shape != dq.shape or dv.shape != dq.shape or dk.dtype != dq.dtype or dv.dtype != dq.dtype:
+        raise ValueError("attn_qkv_conv_pullback: dq, dk, dv must share shape [B, P, H, T, Dh] and dtype")
+    if heads % n_kv_heads:
+        raise ValueError("n_heads must be divisible by n_kv_heads")
+    if head_dim % 2:
+        raise ValueError("RoPE requires an even head dimension.")
+    channels = (heads + 2 * n_kv_heads) * head_dim
+    if conv_weight.dim() != 3 or conv_weight.shape[0] != channels or conv_weight.shape[1] != 1:
+        raise ValueError("attn_qkv_conv_pullback: weight must be [C, 1, k] (depthwise) with C = (H + 2 Hkv) Dh")
+    dq, dk, dv = dq.contiguous(), dk.contiguous(), dv.contiguous()
+    weight = conv_weight.to(dq.dtype).contiguous()
+    cos, sin = rope_tables(seqlen, head_dim, rope_base, dq.device)
+    out = torch.empty((bsz, basis, seqlen, channels), device=dq.device, dtype=dq.dtype)
+    with torch.cuda.device(out.device):
+        status = _lib.load().lbi_attn_qkv_conv_pullback(
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), cos.data_ptr(), sin.data_ptr(), weight.data_ptr(),
+            out.data_ptr(), bsz, basis, seqlen, heads, n_kv_heads, head_dim, int(bool(rope_interleaved)),
+            weight.shape[-1], _lib.dtype_code(out.dtype), _stream(out))
+    _lib.check(status, "lbi_attn_qkv_conv_pullback")
+    return out
+
+
 def _apply_transposed(g: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``g @ weight`` for ``weight [out, in]``: the pullback of ``y = x weight^T``.  Issued as
     the library's ``A B^T`` form on a transposed copy of the (small) weight, which is its faster
@@ -251,17 +283,23 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
     dq, dk, dv = attention_input_pullback_basis(a_cache.q_rope, a_cache.k_expanded, a_cache.v_expanded, g_heads,
                                                 softmax_scale=float(scale), causal=True, kernel_mode=kernel_mode)
     del g_heads
-    g_qkv = attn_qkv_pullback(dq, dk, dv, n_kv_heads=attn.n_kv_heads, rope_base=attn.rope_base,
-                              rope_interleaved=attn.rope_interleaved)
-    del dq, dk, dv
-    if attn.d_conv > 0:
-        if param_grads is not None:
-            # the cache keeps the projection after the convolution only: redo the projection
-            bias = getattr(attn.in_proj, "bias", None)
-            x_pre = torch.nn.functional.linear(a_cache.norm_output, attn.in_proj.weight, bias)
-            _conv_grads(param_grads, attn.conv1d, g_qkv, x_pre)
-            del x_pre
-        g_qkv = causal_conv1d_pullback(g_qkv, attn.conv1d.weight)
+    if attn.d_conv > 0 and param_grads is None and attn.conv1d.weight.shape[-1] <= FUSED_CONV_MAX_TAPS:
+        # nothing needs the cotangent of the convolved projection itself: one pass
+        g_qkv = attn_qkv_conv_pullback(dq, dk, dv, attn.conv1d.weight, n_kv_heads=attn.n_kv_heads,
+                                       rope_base=attn.rope_base, rope_interleaved=attn.rope_interleaved)
+        del dq, dk, dv
+    else:
+        g_qkv = attn_qkv_pullback(dq, dk, dv, n_kv_heads=attn.n_kv_heads, rope_base=attn.rope_base,
+                                  rope_interleaved=attn.rope_interleaved)
+        del dq, dk, dv
+        if attn.d_conv > 0:
+            if param_grads is not None:
+                # the cache keeps the projection after the convolution only: redo the projection
+                bias = getattr(attn.in_proj, "bias", None)
+                x_pre = torch.nn.functional.linear(a_cache.norm_output, attn.in_proj.weight, bias)
+                _conv_grads(param_grads, attn.conv1d, g_qkv, x_pre)
+                del x_pre
+            g_qkv = causal_conv1d_pullback(g_qkv, attn.conv1d.weight)
     if param_grads is not None:
         _linear_grads(param_grads, attn.in_proj, g_qkv, a_cache.norm_output)
     g_norm1 = _apply_transposed(g_qkv, attn.in_proj.weight)
@@ -340,6 +378,6 @@ def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tenso
 
 
 __all__ = [
-    "attn_heads_split", "attn_qkv_pullback", "causal_conv1d_pullback", "gated_mlp_pullback", "rmsnorm_pullback",
+    "attn_heads_split", "attn_qkv_conv_pullback", "attn_qkv_pullback", "causal_conv1d_pullback", "gated_mlp_pullback", "rmsnorm_pullback",
     "region_input_pullback_basis", "region_parameter_vjp", "rope_tables",
 ]

@@ -139,6 +139,51 @@ def test_causal_conv1d_pullback(dtype, channels, ksize, seqlen, device):
     assert _max_rel(got, want) <= (1e-6 if dtype == torch.float32 else _tol(dtype))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,interleaved,ksize,seqlen",
+                         [(4, 2, 8, False, 4, 19), (4, 4, 8, True, 3, 8), (3, 1, 6, False, 4, 5), (3, 1, 2, True, 1, 9),
+                          (12, 4, 64, False, 4, 33), (2, 1, 64, True, 7, 12), (2, 2, 16, False, 8, 3)])
+def test_qkv_conv_pullback_equals_the_two_calls(dtype, heads, kv_heads, head_dim, interleaved, ksize, seqlen, device):
+    """The one-pass projection + convolution pullback repeats the arithmetic of the two kernels it replaces (each
+    of which is checked against autograd above), through run boundaries, sequence ends and grouped heads."""
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(heads * 1000 + head_dim * 10 + ksize)
+    b, p = 2, 3
+    channels = (heads + 2 * kv_heads) * head_dim
+    dq, dk, dv = (torch.randn(b, p, heads, seqlen, head_dim).to(dtype).to(device) for _ in range(3))
+    weight = torch.randn(channels, 1, ksize).to(dtype).to(device)
+    kwargs = dict(n_kv_heads=kv_heads, rope_base=100.0, rope_interleaved=interleaved)
+    want = region.causal_conv1d_pullback(region.attn_qkv_pullback(dq, dk, dv, **kwargs), weight)
+    got = region.attn_qkv_conv_pullback(dq, dk, dv, weight, **kwargs)
+    assert got.dtype == dtype and got.shape == want.shape
+    differing = int((got != want).sum())
+    if dtype == torch.float32:
+        assert differing == 0, f"{differing} elements differ"
+    else:
+        # same arithmetic, but the compiler may fuse a final multiply-add with the narrowing conversion in one
+        # kernel and not in the other: a last-place difference on a few elements in 10^5 is allowed, nothing more
+        ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
+        assert differing <= max(1, got.numel() // 2000), f"{differing} of {got.numel()} elements differ"
+        assert float(((got.float() - want.float()).abs() / want.float().abs().clamp_min(1e-3)).max()) <= ulp
+
+
+def test_qkv_conv_pullback_contract(device):
+    from latent_bounded_interfaces_amd._lib import LbiLibraryError
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    dq = torch.randn(1, 1, 2, 4, 8, device=device)
+    with pytest.raises(ValueError, match="depthwise"):
+        region.attn_qkv_conv_pullback(dq, dq, dq, torch.randn(5, 1, 4, device=device), n_kv_heads=2, rope_base=10.0,
+                                      rope_interleaved=False)
+    with pytest.raises(LbiLibraryError, match="above 8"):
+        region.attn_qkv_conv_pullback(dq, dq, dq, torch.randn(48, 1, 9, device=device), n_kv_heads=2, rope_base=10.0,
+                                      rope_interleaved=False)
+    with pytest.raises(RuntimeError, match="no CPU execution path"):
+        region.attn_qkv_conv_pullback(dq.cpu(), dq.cpu(), dq.cpu(), torch.randn(48, 1, 4), n_kv_heads=2,
+                                      rope_base=10.0, rope_interleaved=False)
+
+
 REGION_CASES = [
     # dim, heads, kv, head_dim, hidden, layers, d_conv, interleaved, B, P, T
     (32, 4, 2, 8, 48, 2, 4, False, 2, 3, 12),
