@@ -208,6 +208,23 @@ int lbi_attn_qkv_conv_pullback(const void* dq, const void* dk, const void* dv,
                                void* g_in, int64_t B, int64_t P, int64_t T, int64_t H, int64_t Hkv,
                                int64_t Dh, int interleaved, int64_t ksize, int dtype, void* stream);
 
+/*
+ * Frobenius and spectral (largest singular value) norms of N square matrices, the per-step Jacobian
+ * diagnostics of the interface scan (reference backward/suffix_scan.py:105-134, which calls
+ * torch.linalg.matrix_norm with ord="fro" and ord=2, a singular value decomposition per matrix).
+ *
+ *   mats [N,d,d] (dtype)  ->  spectral [N], frobenius [N]   (fp32)
+ *
+ * No decomposition: the top eigenvalue of A^T A comes from repeated squaring with the trace divided
+ * out, at most 24 squarings, which bounds the relative error by 2^-25 log(d) plus fp32 rounding for
+ * any spectrum.  `workspace` must hold lbi_matrix_norms_workspace_bytes(N, d) bytes (0 for d <= 88,
+ * whose buffers fit in LDS), 16-byte aligned.  d <= 2048.
+ */
+size_t lbi_matrix_norms_workspace_bytes(int64_t N, int64_t d);
+int lbi_matrix_norms(const void* mats, float* spectral, float* frobenius,
+                     void* workspace, size_t workspace_bytes,
+                     int64_t N, int64_t d, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

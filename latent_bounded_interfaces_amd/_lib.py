@@ -14,7 +14,7 @@ import torch
 LIB_PATH = Path(__file__).resolve().parent / "liblbi_hip.so"
 
 LBI_F32, LBI_F16, LBI_BF16 = 0, 1, 2
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _DTYPE_CODES = {torch.float32: LBI_F32, torch.float16: LBI_F16, torch.bfloat16: LBI_BF16}
 
@@ -59,6 +59,11 @@ SYMBOLS = {
     "lbi_attn_qkv_conv_pullback": (
         _c.c_int,
         [_c.c_void_p] * 7 + [_c.c_int64] * 6 + [_c.c_int, _c.c_int64, _c.c_int, _c.c_void_p],
+    ),
+    "lbi_matrix_norms_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64]),
+    "lbi_matrix_norms": (
+        _c.c_int,
+        [_c.c_void_p] * 4 + [_c.c_size_t, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p],
     ),
 }
 

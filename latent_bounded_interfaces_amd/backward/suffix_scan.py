@@ -10,7 +10,7 @@ from collections.abc import Sequence
 
 import torch
 
-from ..hip.interface import suffix_scan_cotangents
+from ..hip.interface import matrix_norms, suffix_scan_cotangents
 from ..hip.interface import suffix_scan_pullbacks as suffix_scan_jacobian_t
 
 
@@ -120,28 +120,23 @@ def interface_state_jacobian_t_stats(
     *,
     include_suffix: bool,
 ) -> dict[str, float]:
-    """Frobenius / spectral norm diagnostics (reference backward/suffix_scan.py:105-134)."""
+    """Frobenius / spectral norm diagnostics (reference backward/suffix_scan.py:105-134): same keys and
+    values, from one ``lbi_matrix_norms`` launch per group of matrices instead of a singular value
+    decomposition per matrix; the only host synchronisation is the final read of the seven scalars."""
     if not state_jacobians_t:
         return {}
     with torch.no_grad():
-        dense = torch.stack([jt.detach().float() for jt in state_jacobians_t], dim=1)
-        frob = torch.linalg.matrix_norm(dense, ord="fro", dim=(-2, -1))
-        spec = torch.linalg.matrix_norm(dense, ord=2, dim=(-2, -1))
+        dense = torch.stack([jt.detach() for jt in state_jacobians_t], dim=1)
+        if dense.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+            dense = dense.float()
+        spec, frob = matrix_norms(dense)
         rank = max(1, int(dense.shape[-1]))
-        stats = {
-            "jac_local_spec_mean": float(spec.mean().item()),
-            "jac_local_spec_max": float(spec.max().item()),
-            "jac_local_frob_mean": float(frob.mean().item()),
-            "jac_local_frob_max": float(frob.max().item()),
-            "jac_local_frob_normed_mean": float((frob / (rank ** 0.5)).mean().item()),
-        }
+        values = [spec.mean(), spec.max(), frob.mean(), frob.max(), (frob / (rank ** 0.5)).mean()]
+        keys = ["jac_local_spec_mean", "jac_local_spec_max", "jac_local_frob_mean", "jac_local_frob_max",
+                "jac_local_frob_normed_mean"]
         if include_suffix:
-            suffix = suffix_scan_jacobian_t(dense.contiguous())
-            suffix_spec = torch.linalg.matrix_norm(suffix, ord=2, dim=(-2, -1))
-            stats.update(
-                {
-                    "jac_suffix_spec_mean": float(suffix_spec.mean().item()),
-                    "jac_suffix_spec_max": float(suffix_spec.max().item()),
-                }
-            )
-        return stats
+            suffix_spec, _ = matrix_norms(suffix_scan_jacobian_t(dense.contiguous()))
+            values += [suffix_spec.mean(), suffix_spec.max()]
+            keys += ["jac_suffix_spec_mean", "jac_suffix_spec_max"]
+        host = torch.stack(values).cpu().tolist()
+        return dict(zip(keys, (float(v) for v in host)))

@@ -92,4 +92,39 @@ def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor) ->
     return out, cot
 
 
-__all__ = ["suffix_scan_pullbacks", "suffix_scan_cotangents", "suffix_scan_pullbacks_and_cotangents"]
+def matrix_norms(mats: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(spectral, frobenius)`` norms, fp32, of every square matrix of ``mats [..., d, d]``.
+
+    What reference backward/suffix_scan.py:117-118 and :126 get from ``torch.linalg.matrix_norm``
+    (``ord=2`` runs a singular value decomposition per matrix); here one ``lbi_matrix_norms`` launch
+    (repeated squaring of ``A^T A``, no decomposition).
+    """
+    if not isinstance(mats, torch.Tensor):
+        raise TypeError("mats must be a torch.Tensor")
+    if mats.dim() < 2 or mats.shape[-1] != mats.shape[-2]:
+        raise ValueError("mats must be square in the last two dimensions")
+    if not mats.is_cuda:
+        raise RuntimeError("mats must be a CUDA tensor (this build has no CPU execution path)")
+    if mats.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        raise RuntimeError("mats must have float, half, or bfloat16 dtype")
+    batch_shape = mats.shape[:-2]
+    rank = int(mats.shape[-1])
+    mats = mats.contiguous()
+    count = mats.numel() // (rank * rank) if rank else 0
+    spectral = torch.empty(batch_shape, device=mats.device, dtype=torch.float32)
+    frobenius = torch.empty(batch_shape, device=mats.device, dtype=torch.float32)
+    if count == 0:
+        return spectral, frobenius
+    lib = _lib.load()
+    need = int(lib.lbi_matrix_norms_workspace_bytes(count, rank))
+    workspace = torch.empty(max(need, 16), device=mats.device, dtype=torch.uint8)
+    with torch.cuda.device(mats.device):
+        status = lib.lbi_matrix_norms(
+            mats.data_ptr(), spectral.data_ptr(), frobenius.data_ptr(), workspace.data_ptr(), workspace.numel(),
+            count, rank, _lib.dtype_code(mats.dtype), _lib.current_stream_ptr(mats.device),
+        )
+    _lib.check(status, "lbi_matrix_norms")
+    return spectral, frobenius
+
+
+__all__ = ["matrix_norms", "suffix_scan_pullbacks", "suffix_scan_cotangents", "suffix_scan_pullbacks_and_cotangents"]

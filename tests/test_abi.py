@@ -50,6 +50,33 @@ def test_argument_validation_needs_no_gpu():
     assert lib.lbi_suffix_cotangents(None, None, None, 1, 2, 4, _lib.LBI_F32, None) == -1
 
 
+def test_region_and_norm_entry_points_validate_on_the_host():
+    lib = _lib.load()
+    f32 = _lib.LBI_F32
+    assert lib.lbi_rmsnorm_pullback(None, None, None, None, None, None, 1, 1, 1, 8, 1e-5, f32, f32, None) == -1
+    assert b"null" in lib.lbi_last_error()
+    assert lib.lbi_gated_mlp_pullback(None, None, None, 1, 1, 1, 8, 9, None) == -1
+    assert lib.lbi_attn_heads_split(None, None, 1, 1, 1, 1, 8, f32, None) == -1
+    one = ctypes.c_void_p(256)  # never dereferenced: every call below is rejected before any launch
+    assert lib.lbi_attn_qkv_pullback(one, one, one, one, one, one, 1, 1, 4, 3, 2, 8, 0, f32, None) == -1
+    assert b"multiple" in lib.lbi_last_error()
+    assert lib.lbi_attn_qkv_conv_pullback(one, one, one, one, one, one, one, 1, 1, 4, 2, 2, 7, 0, 4, f32, None) == -1
+    assert b"even head dim" in lib.lbi_last_error()
+    assert lib.lbi_attn_qkv_conv_pullback(one, one, one, one, one, one, one, 1, 1, 4, 2, 2, 8, 0, 9, f32, None) == -2
+    assert b"above 8" in lib.lbi_last_error()
+    assert lib.lbi_causal_conv1d_pullback(one, one, one, 1, 4, 8, 4, f32, None) == -1
+    assert b"in-place" in lib.lbi_last_error()
+    # spectral / Frobenius norms: LDS-resident sizes need no workspace, larger ones two planes per workgroup
+    assert lib.lbi_matrix_norms_workspace_bytes(10, 64) == 0
+    assert lib.lbi_matrix_norms_workspace_bytes(10, 88) == 0
+    assert lib.lbi_matrix_norms_workspace_bytes(10, 90) == 10 * 2 * 92 * 92 * 4
+    assert lib.lbi_matrix_norms_workspace_bytes(5000, 256) == 1024 * 2 * 256 * 256 * 4
+    assert lib.lbi_matrix_norms(one, one, one, None, 0, 4, 0, f32, None) == -1
+    assert lib.lbi_matrix_norms(one, one, one, None, 0, 4, 256, f32, None) == -4
+    assert b"workspace" in lib.lbi_last_error()
+    assert lib.lbi_matrix_norms(None, None, None, None, 0, 0, 16, f32, None) == 0
+
+
 def test_wrappers_reject_bad_input_before_touching_the_device():
     import torch
 
