@@ -138,25 +138,30 @@ int lbi_attn_pullback(const void* q, const void* k, const void* v, const void* d
  *   residual stream, reference backends/transformer.py:197,201);
  *   g_residual [B,P,T,D] fp32 or NULL; outputs g_sum [B,P,T,D] fp32 and/or g_sum_branch
  *   [B,P,T,D] branch_dtype (either may be NULL, not both).  g_sum may alias g_residual.
+ *   g_residual_broadcast_t != 0: g_residual is [B,P,D], the same for every position (the
+ *   cotangent a mean-pooling interface sends into the region output, reference
+ *   interfaces/vector_mlp.py:111-116); it then must not alias g_sum.
  *   Forward: RMSNorm.forward, reference backbones/transformer/block.py:12-23, applied by
  *   TransformerBlock._prenorm (block.py:66-76).
  */
 int lbi_rmsnorm_pullback(const void* g_out, const void* x, const void* weight, const void* g_residual,
                          void* g_sum, void* g_sum_branch,
                          int64_t B, int64_t P, int64_t T, int64_t D, float eps,
-                         int branch_dtype, int x_dtype, void* stream);
+                         int g_residual_broadcast_t, int branch_dtype, int x_dtype, void* stream);
 
 /*
  * Gated-MLP pullback through  down_input = up * silu(gate),  [up | gate] = fc1_output.
  *
  *   g_down_input [B,P,T,hidden], fc1_output [B,T,2*hidden]  ->  g_fc1_output [B,P,T,2*hidden]
  *   g_up = g * silu(gate);   g_gate = g * up * silu'(gate)
+ *   g_broadcast_t != 0: g_down_input is [B,P,hidden], the same for every position.
  *
  * Forward: reference backends/transformer.py:172-176 (GatedMLP.forward,
  * backbones/transformer/mlp.py:30-32).
  */
 int lbi_gated_mlp_pullback(const void* g_down_input, const void* fc1_output, void* g_fc1_output,
-                           int64_t B, int64_t P, int64_t T, int64_t hidden, int dtype, void* stream);
+                           int64_t B, int64_t P, int64_t T, int64_t hidden,
+                           int g_broadcast_t, int dtype, void* stream);
 
 /*
  * Head split of the out_proj-input cotangent: [B,P,T,H*Dh] -> [B,P,H,T,Dh], the layout

@@ -14,7 +14,7 @@ import torch
 LIB_PATH = Path(__file__).resolve().parent / "liblbi_hip.so"
 
 LBI_F32, LBI_F16, LBI_BF16 = 0, 1, 2
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _DTYPE_CODES = {torch.float32: LBI_F32, torch.float16: LBI_F16, torch.bfloat16: LBI_BF16}
 
@@ -47,9 +47,9 @@ SYMBOLS = {
     ),
     "lbi_rmsnorm_pullback": (
         _c.c_int,
-        [_c.c_void_p] * 6 + [_c.c_int64] * 4 + [_c.c_float, _c.c_int, _c.c_int, _c.c_void_p],
+        [_c.c_void_p] * 6 + [_c.c_int64] * 4 + [_c.c_float, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p],
     ),
-    "lbi_gated_mlp_pullback": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_int64] * 4 + [_c.c_int, _c.c_void_p]),
+    "lbi_gated_mlp_pullback": (_c.c_int, [_c.c_void_p] * 3 + [_c.c_int64] * 4 + [_c.c_int, _c.c_int, _c.c_void_p]),
     "lbi_attn_heads_split": (_c.c_int, [_c.c_void_p] * 2 + [_c.c_int64] * 5 + [_c.c_int, _c.c_void_p]),
     "lbi_attn_qkv_pullback": (
         _c.c_int,

@@ -32,11 +32,33 @@ class StructuredInterfacePullbackProvider:
 
     name = "structured"
 
-    def __init__(self, *, basis_chunk: int = 0) -> None:
+    def __init__(self, *, basis_chunk: int = 0, position_constant_update: str = "verify_once") -> None:
         # directions pulled back per call; 0 = all d at once
         if int(basis_chunk) < 0:
             raise ValueError("basis_chunk must be >= 0.")
+        if position_constant_update not in {"verify_once", "verify", "off"}:
+            raise ValueError("position_constant_update must be one of: verify_once, verify, off")
         self.basis_chunk = int(basis_chunk)
+        self.position_constant_update = position_constant_update
+        self._constant_over_positions: dict[type, bool] = {}
+
+    def _region_output_cotangent(self, interface: Any, g_region_output: torch.Tensor) -> torch.Tensor:
+        """An interface that pools the region output with a mean over positions sends the same cotangent to
+        every position (reference interfaces/vector_mlp.py:111-116 materialises it as a dense [B,P,T,D]
+        tensor).  When that holds the tensor is handed on as a stride-0 view of its first position, which lets
+        the region pullback run the last block's first product on one row per direction.  Whether it holds is
+        a property of the interface class: it is checked on the device (one host synchronisation) the first
+        time a class is seen (``verify_once``), on every call (``verify``), or never used (``off``)."""
+        if self.position_constant_update == "off" or g_region_output.dim() != 4 or g_region_output.shape[2] <= 1:
+            return g_region_output
+        if g_region_output.stride(2) == 0:
+            return g_region_output
+        first = g_region_output[:, :, :1].expand_as(g_region_output)
+        known = self._constant_over_positions.get(type(interface)) if self.position_constant_update == "verify_once" else None
+        if known is None:
+            known = bool(torch.equal(first, g_region_output))
+            self._constant_over_positions[type(interface)] = known
+        return first if known else g_region_output
 
     def region_state_jacobian_t(self, *, model: Any, region_cache: Any) -> torch.Tensor:
         state_in = region_cache.state_in
@@ -51,8 +73,9 @@ class StructuredInterfacePullbackProvider:
                 basis = eye[start:start + chunk].unsqueeze(0).expand(bsz, -1, rank)
                 update = model.interface.apply_update_jacobian_t_to_region_output(
                     region_cache=region_cache, state_out_cotangent_basis=basis)
+                g_region_output = self._region_output_cotangent(model.interface, update["g_region_output"])
                 g_region_input = model.region_backend.input_pullback_basis(
-                    cache=region_cache.backend_cache, output_cotangent_basis=update["g_region_output"])
+                    cache=region_cache.backend_cache, output_cotangent_basis=g_region_output)
                 decode = model.interface.apply_decode_jacobian_t_to_state_input(
                     region_cache=region_cache, region_input_cotangent_basis=g_region_input)
                 total = update["g_state_skip"] + decode["g_state_input"]  # [B, P, d_in]
@@ -66,10 +89,12 @@ class StructuredInterfacePullbackProvider:
         return [self.region_state_jacobian_t(model=model, region_cache=rc) for rc in region_caches]
 
 
-def build_interface_pullback_provider(mode: str, *, basis_chunk: int = 0) -> StructuredInterfacePullbackProvider:
+def build_interface_pullback_provider(mode: str, *, basis_chunk: int = 0,
+                                      position_constant_update: str = "verify_once") -> StructuredInterfacePullbackProvider:
     """Name lookup in the style of reference backward/pullbacks.py:185-197; the autograd
     providers of the reference stay in the reference."""
     normalized = str(mode).strip().lower().replace("-", "_")
     if normalized in {"structured", "hip", "structured_hip"}:
-        return StructuredInterfacePullbackProvider(basis_chunk=basis_chunk)
+        return StructuredInterfacePullbackProvider(basis_chunk=basis_chunk,
+                                                   position_constant_update=position_constant_update)
     raise ValueError("interface pullback provider must be one of: structured, hip")

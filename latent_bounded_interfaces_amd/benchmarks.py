@@ -240,7 +240,8 @@ def measure_lbi_step(*, regions=6, layers_per_region=2, dim=768, n_heads=12, hea
     """Device work of one LBI scan backward step at the end-to-end configuration (12 layers in 6
     regions of 2, interface width 64): per region the state-Jacobian build (region input pullback
     for 64 directions) and the parameter VJP, then the interface suffix scan (cotangent chain over
-    the 5 inner Jacobians).  The forward caches are synthetic and shared by the six regions
+    the 5 inner Jacobians).  The region-output cotangents are constant over positions (mean-pooling
+    interface).  The forward caches are synthetic and shared by the six regions
     (same shapes); the interface's own small MLP pullbacks and the readout/canvas VJPs are not part
     of this library and are left out."""
     from .backends import HipTransformerLowering
@@ -250,7 +251,9 @@ def measure_lbi_step(*, regions=6, layers_per_region=2, dim=768, n_heads=12, hea
                                       layers=layers_per_region, d_conv=d_conv, batch=batch, seq_len=seq_len,
                                       dtype=dtype, device=device)
     gen = torch.Generator(device="cpu").manual_seed(2)
-    basis = (torch.randn(batch, interface_width, 1, dim, generator=gen) / seq_len).expand(-1, -1, seq_len, -1).to(device)
+    # what the structured provider hands over for a mean-pooling interface: one cotangent per direction,
+    # the same at every position, as a stride-0 view
+    basis = (torch.randn(batch, interface_width, 1, dim, generator=gen) / seq_len).to(device).expand(-1, -1, seq_len, -1)
     cot = torch.randn(batch, seq_len, dim, generator=gen).to(device)
     jts = (torch.eye(interface_width) + 0.05 * torch.randn(batch, regions - 1, interface_width, interface_width,
                                                           generator=gen)).to(device)

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void rmsnorm_pullback_kernel(const TB* __restr
                                                                const TB* __restrict__ weight,
                                                                const float* g_residual, float* g_sum,
                                                                TB* __restrict__ g_sum_branch, long long n_rows,
-                                                               int P, int T_len, int D, float eps) {
+                                                               int P, int T_len, int D, float eps, int res_bcast) {
     const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= n_rows) return;
     const int lane = threadIdx.x & 63;
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void rmsnorm_pullback_kernel(const TB* __restr
         g.load(g_row + j);
         w.load(weight + j);
         xv.load(x_row + j);
-        if (g_residual != nullptr) res.load(g_residual + row * D + j);
+        if (g_residual != nullptr) res.load(g_residual + (res_bcast ? bp : row) * D + j);  // [B,P,D] or [B,P,T,D]
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const float xr = round_via<TB>(xv.v[i]);
@@ -161,7 +161,7 @@ template <typename T, int VEC>
 __global__ __launch_bounds__(256) void gated_mlp_pullback_kernel(const T* __restrict__ g_down_input,
                                                                  const T* __restrict__ fc1_output,
                                                                  T* __restrict__ g_fc1_output, int P, int T_len,
-                                                                 int hidden) {
+                                                                 int hidden, int g_bcast) {
     const int b = blockIdx.x / T_len, t = blockIdx.x - b * T_len;
     const T* act_row = fc1_output + (long long)blockIdx.x * 2 * hidden;
     const long long row0 = (long long)b * P * T_len + t;  // cotangent row of direction 0
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) void gated_mlp_pullback_kernel(const T* __rest
         for (int p = 0; p < P; ++p) {
             const long long row = row0 + (long long)p * T_len;
             Pack<T, VEC> g, o_up, o_gate;
-            g.load(g_down_input + row * hidden + j);
+            g.load(g_down_input + (g_bcast ? (long long)b * P + p : row) * hidden + j);  // [B,P,hidden] or [B,P,T,hidden]
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
                 o_up.v[i] = g.v[i] * act[i];
@@ -517,16 +517,17 @@ inline bool fits_grid(long long units, int per_block) {
 
 template <typename TB, typename TX>
 int launch_rmsnorm(const void* g_out, const void* x, const void* weight, const void* g_residual, void* g_sum,
-                   void* g_sum_branch, long long n_rows, int P, int T_len, int D, float eps, hipStream_t stream) {
+                   void* g_sum_branch, long long n_rows, int P, int T_len, int D, float eps, int res_bcast,
+                   hipStream_t stream) {
     const dim3 grid(blocks_for(n_rows, 4)), block(256);
     if (D % 4 == 0)
         hipLaunchKernelGGL((rmsnorm_pullback_kernel<TB, TX, 4>), grid, block, 0, stream, (const TB*)g_out, (const TX*)x,
                            (const TB*)weight, (const float*)g_residual, (float*)g_sum, (TB*)g_sum_branch, n_rows, P,
-                           T_len, D, eps);
+                           T_len, D, eps, res_bcast);
     else
         hipLaunchKernelGGL((rmsnorm_pullback_kernel<TB, TX, 1>), grid, block, 0, stream, (const TB*)g_out, (const TX*)x,
                            (const TB*)weight, (const float*)g_residual, (float*)g_sum, (TB*)g_sum_branch, n_rows, P,
-                           T_len, D, eps);
+                           T_len, D, eps, res_bcast);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
@@ -534,35 +535,35 @@ int launch_rmsnorm(const void* g_out, const void* x, const void* weight, const v
 template <typename TB>
 int launch_rmsnorm_x(int x_dtype, const void* g_out, const void* x, const void* weight, const void* g_residual,
                      void* g_sum, void* g_sum_branch, long long n_rows, int P, int T_len, int D, float eps,
-                     hipStream_t stream) {
+                     int res_bcast, hipStream_t stream) {
     switch (x_dtype) {
-        case LBI_F32: return launch_rmsnorm<TB, float>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, stream);
-        case LBI_F16: return launch_rmsnorm<TB, _Float16>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, stream);
-        default: return launch_rmsnorm<TB, bf16_raw>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, stream);
+        case LBI_F32: return launch_rmsnorm<TB, float>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, res_bcast, stream);
+        case LBI_F16: return launch_rmsnorm<TB, _Float16>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, res_bcast, stream);
+        default: return launch_rmsnorm<TB, bf16_raw>(g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, P, T_len, D, eps, res_bcast, stream);
     }
 }
 
 template <typename T, int VEC>
 int launch_gated_as(const void* g, const void* fc1, void* out, long long n_tokens, int P, int T_len, int hidden,
-                    hipStream_t stream) {
+                    int g_bcast, hipStream_t stream) {
     if (n_tokens > 0x7fffffffLL) return fail(LBI_ERR_UNSUPPORTED, "lbi_gated_mlp_pullback: too many tokens");
     const int chunks = hidden / VEC;
     const int threads = chunks >= 256 ? 256 : ((chunks + 63) / 64) * 64;
     hipLaunchKernelGGL((gated_mlp_pullback_kernel<T, VEC>), dim3((unsigned)n_tokens), dim3(threads), 0, stream,
-                       (const T*)g, (const T*)fc1, (T*)out, P, T_len, hidden);
+                       (const T*)g, (const T*)fc1, (T*)out, P, T_len, hidden, g_bcast);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
 
 template <typename T>
 int launch_gated(const void* g, const void* fc1, void* out, long long n_rows, int P, int T_len, int hidden,
-                 hipStream_t stream) {  // n_rows: tokens B * T
+                 int g_bcast, hipStream_t stream) {  // n_rows: tokens B * T
     constexpr int W = wide<T>();
     const bool aligned =
         (reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(fc1) | reinterpret_cast<uintptr_t>(out)) % 16 == 0;
-    if (hidden % W == 0 && aligned) return launch_gated_as<T, W>(g, fc1, out, n_rows, P, T_len, hidden, stream);
-    if (hidden % 4 == 0 && sizeof(T) == 4) return launch_gated_as<T, 4>(g, fc1, out, n_rows, P, T_len, hidden, stream);
-    return launch_gated_as<T, 1>(g, fc1, out, n_rows, P, T_len, hidden, stream);
+    if (hidden % W == 0 && aligned) return launch_gated_as<T, W>(g, fc1, out, n_rows, P, T_len, hidden, g_bcast, stream);
+    if (hidden % 4 == 0 && sizeof(T) == 4) return launch_gated_as<T, 4>(g, fc1, out, n_rows, P, T_len, hidden, g_bcast, stream);
+    return launch_gated_as<T, 1>(g, fc1, out, n_rows, P, T_len, hidden, g_bcast, stream);
 }
 
 template <typename T>
@@ -665,7 +666,8 @@ using namespace lbi;
 
 extern "C" int lbi_rmsnorm_pullback(const void* g_out, const void* x, const void* weight, const void* g_residual,
                                     void* g_sum, void* g_sum_branch, int64_t B, int64_t P, int64_t T, int64_t D,
-                                    float eps, int branch_dtype, int x_dtype, void* stream) {
+                                    float eps, int g_residual_broadcast_t, int branch_dtype, int x_dtype,
+                                    void* stream) {
     clear_error();
     if (!g_out || !x || !weight) return fail(LBI_ERR_INVALID, "lbi_rmsnorm_pullback: null input pointer");
     if (!g_sum && !g_sum_branch) return fail(LBI_ERR_INVALID, "lbi_rmsnorm_pullback: no output requested");
@@ -677,16 +679,20 @@ extern "C" int lbi_rmsnorm_pullback(const void* g_out, const void* x, const void
     const long long n_rows = (long long)B * P * T;
     if (n_rows == 0) return LBI_OK;
     if (!region::fits_grid(n_rows, 4)) return fail(LBI_ERR_UNSUPPORTED, "lbi_rmsnorm_pullback: too many rows");
+    if (g_residual_broadcast_t && g_sum == g_residual)
+        return fail(LBI_ERR_INVALID, "lbi_rmsnorm_pullback: a residual shared over T cannot be updated in place");
+    const int rb = g_residual_broadcast_t != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (branch_dtype) {
-        case LBI_F32: return region::launch_rmsnorm_x<float>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, s);
-        case LBI_F16: return region::launch_rmsnorm_x<_Float16>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, s);
-        default: return region::launch_rmsnorm_x<bf16_raw>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, s);
+        case LBI_F32: return region::launch_rmsnorm_x<float>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, rb, s);
+        case LBI_F16: return region::launch_rmsnorm_x<_Float16>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, rb, s);
+        default: return region::launch_rmsnorm_x<bf16_raw>(x_dtype, g_out, x, weight, g_residual, g_sum, g_sum_branch, n_rows, (int)P, (int)T, (int)D, eps, rb, s);
     }
 }
 
 extern "C" int lbi_gated_mlp_pullback(const void* g_down_input, const void* fc1_output, void* g_fc1_output, int64_t B,
-                                      int64_t P, int64_t T, int64_t hidden, int dtype, void* stream) {
+                                      int64_t P, int64_t T, int64_t hidden, int g_broadcast_t, int dtype,
+                                      void* stream) {
     clear_error();
     if (!g_down_input || !fc1_output || !g_fc1_output)
         return fail(LBI_ERR_INVALID, "lbi_gated_mlp_pullback: null pointer");
@@ -697,9 +703,9 @@ extern "C" int lbi_gated_mlp_pullback(const void* g_down_input, const void* fc1_
     const long long n_rows = (long long)B * T;  // one workgroup per token
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
-        case LBI_F32: return region::launch_gated<float>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, s);
-        case LBI_F16: return region::launch_gated<_Float16>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, s);
-        default: return region::launch_gated<bf16_raw>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, s);
+        case LBI_F32: return region::launch_gated<float>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, g_broadcast_t != 0, s);
+        case LBI_F16: return region::launch_gated<_Float16>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, g_broadcast_t != 0, s);
+        default: return region::launch_gated<bf16_raw>(g_down_input, fc1_output, g_fc1_output, n_rows, (int)P, (int)T, (int)hidden, g_broadcast_t != 0, s);
     }
 }
 

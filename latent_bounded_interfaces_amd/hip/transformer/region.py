@@ -42,42 +42,56 @@ def rmsnorm_pullback(g_out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor,
                      g_residual: torch.Tensor | None, *, want_branch: bool) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``g_out [B,P,T,D]`` through RMSNorm at input ``x [B,T,D]``, plus ``g_residual`` (fp32).
 
-    Returns ``(sum fp32, sum in g_out.dtype or None)``.  ``g_residual`` is overwritten with the sum.
+    Returns ``(sum fp32, sum in g_out.dtype or None)``.  ``g_residual [B,P,T,D]`` is overwritten with the
+    sum; ``g_residual [B,P,1,D]`` (the same cotangent at every position) is read only.
     """
     _require_cuda(g_out, x, weight)
     bsz, basis, seqlen, dim = g_out.shape
     if x.shape != (bsz, seqlen, dim) or weight.shape != (dim,):
         raise ValueError("rmsnorm_pullback: x must be [B, T, D] and weight [D] matching g_out [B, P, T, D]")
     g_out, x, weight = g_out.contiguous(), x.contiguous(), weight.to(g_out.dtype).contiguous()
+    shared = 0
     if g_residual is None:
         total = torch.empty(g_out.shape, device=g_out.device, dtype=torch.float32)
         res_ptr = None
     else:
-        if g_residual.dtype != torch.float32 or g_residual.shape != g_out.shape or not g_residual.is_contiguous():
-            raise ValueError("rmsnorm_pullback: g_residual must be a contiguous fp32 tensor shaped like g_out")
-        total = g_residual
+        if g_residual.dtype != torch.float32 or not g_residual.is_contiguous():
+            raise ValueError("rmsnorm_pullback: g_residual must be a contiguous fp32 tensor")
+        if g_residual.shape == g_out.shape:
+            total = g_residual
+        elif g_residual.shape == (bsz, basis, 1, dim):
+            total = torch.empty(g_out.shape, device=g_out.device, dtype=torch.float32)
+            shared = 1
+        else:
+            raise ValueError("rmsnorm_pullback: g_residual must be shaped like g_out, or [B, P, 1, D]")
         res_ptr = g_residual.data_ptr()
     branch = torch.empty_like(g_out) if want_branch else None
     with torch.cuda.device(g_out.device):
         status = _lib.load().lbi_rmsnorm_pullback(
             g_out.data_ptr(), x.data_ptr(), weight.data_ptr(), res_ptr, total.data_ptr(),
-            branch.data_ptr() if branch is not None else None, bsz, basis, seqlen, dim, float(eps),
+            branch.data_ptr() if branch is not None else None, bsz, basis, seqlen, dim, float(eps), shared,
             _lib.dtype_code(g_out.dtype), _lib.dtype_code(x.dtype), _stream(g_out))
     _lib.check(status, "lbi_rmsnorm_pullback")
     return total, branch
 
 
 def gated_mlp_pullback(g_down_input: torch.Tensor, fc1_output: torch.Tensor) -> torch.Tensor:
-    """``g_down_input [B,P,T,Hd]``, ``fc1_output [B,T,2Hd]`` -> cotangent of fc1_output ``[B,P,T,2Hd]``."""
+    """``g_down_input [B,P,T,Hd]`` (or ``[B,P,1,Hd]``: the same at every position), ``fc1_output [B,T,2Hd]``
+    -> cotangent of fc1_output ``[B,P,T,2Hd]``."""
     _require_cuda(g_down_input, fc1_output)
-    bsz, basis, seqlen, hidden = g_down_input.shape
-    if fc1_output.shape != (bsz, seqlen, 2 * hidden) or fc1_output.dtype != g_down_input.dtype:
+    bsz, basis, g_len, hidden = g_down_input.shape
+    if fc1_output.dim() != 3 or fc1_output.shape[0] != bsz or fc1_output.shape[2] != 2 * hidden \
+            or fc1_output.dtype != g_down_input.dtype:
         raise ValueError("gated_mlp_pullback: fc1_output must be [B, T, 2*hidden] in the dtype of g_down_input")
+    seqlen = int(fc1_output.shape[1])
+    if g_len != seqlen and g_len != 1:
+        raise ValueError("gated_mlp_pullback: g_down_input must be [B, P, T, hidden] or [B, P, 1, hidden]")
+    shared = int(g_len == 1 and seqlen != 1)
     g_down_input, fc1_output = g_down_input.contiguous(), fc1_output.contiguous()
     out = torch.empty((bsz, basis, seqlen, 2 * hidden), device=g_down_input.device, dtype=g_down_input.dtype)
     with torch.cuda.device(out.device):
         status = _lib.load().lbi_gated_mlp_pullback(
-            g_down_input.data_ptr(), fc1_output.data_ptr(), out.data_ptr(), bsz, basis, seqlen, hidden,
+            g_down_input.data_ptr(), fc1_output.data_ptr(), out.data_ptr(), bsz, basis, seqlen, hidden, shared,
             _lib.dtype_code(out.dtype), _stream(out))
     _lib.check(status, "lbi_gated_mlp_pullback")
     return out
@@ -241,7 +255,8 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
                           kernel_mode: str, want_branch: bool,
                           param_grads: dict | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
     """One block, backwards.  ``g_residual`` (fp32, [B,P,T,D]) is the cotangent of the block's
-    residual output and is updated in place; ``g_hidden`` is the cotangent of its hidden output
+    residual output and is updated in place (``[B,P,1,D]``: the same at every position, read only);
+    ``g_hidden`` is the cotangent of its hidden output
     in the weight dtype (``None``: equal to ``g_residual``).  Returns the cotangent of
     ``hidden (+ residual)`` at the block input in fp32 and, if ``want_branch``, also rounded to
     the weight dtype (the ``g_hidden`` of the block before).
@@ -315,7 +330,12 @@ def _pull_back_region(backend: Any, cache: Any, cotangent: torch.Tensor, kernel_
     start, end = cache.layer_range
     device = cache.region_input.device
     # region_output = hidden + residual of the last block: both receive the cotangent
-    g = cotangent.to(device=device, dtype=torch.float32, copy=True).contiguous()
+    if param_grads is None and cotangent.shape[2] > 1 and cotangent.stride(2) == 0:
+        # an expanded view: the same cotangent at every position (what mean pooling sends back).  The last
+        # block's down-projection product then runs on one row per (b, p) and the kernels read [B,P,1,*].
+        g = cotangent[:, :, :1].to(device=device, dtype=torch.float32, copy=True).contiguous()
+    else:
+        g = cotangent.to(device=device, dtype=torch.float32, copy=True).contiguous()
     g_branch = None
     for offset in range(end - start - 1, -1, -1):
         layer_cache = cache.layer_caches[offset]

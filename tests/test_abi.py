@@ -53,9 +53,9 @@ def test_argument_validation_needs_no_gpu():
 def test_region_and_norm_entry_points_validate_on_the_host():
     lib = _lib.load()
     f32 = _lib.LBI_F32
-    assert lib.lbi_rmsnorm_pullback(None, None, None, None, None, None, 1, 1, 1, 8, 1e-5, f32, f32, None) == -1
+    assert lib.lbi_rmsnorm_pullback(None, None, None, None, None, None, 1, 1, 1, 8, 1e-5, 0, f32, f32, None) == -1
     assert b"null" in lib.lbi_last_error()
-    assert lib.lbi_gated_mlp_pullback(None, None, None, 1, 1, 1, 8, 9, None) == -1
+    assert lib.lbi_gated_mlp_pullback(None, None, None, 1, 1, 1, 8, 0, 9, None) == -1
     assert lib.lbi_attn_heads_split(None, None, 1, 1, 1, 1, 8, f32, None) == -1
     one = ctypes.c_void_p(256)  # never dereferenced: every call below is rejected before any launch
     assert lib.lbi_attn_qkv_pullback(one, one, one, one, one, one, 1, 1, 4, 3, 2, 8, 0, f32, None) == -1

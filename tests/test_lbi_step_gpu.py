@@ -33,6 +33,40 @@ def test_structured_jacobians_match_graph_provider(basis_chunk, device):
         assert float((a - b).abs().max()) <= 2e-5 * float(b.abs().max()), float((a - b).abs().max())
 
 
+def test_position_constant_update_is_detected_and_optional(device):
+    """The mean-pooling interface sends one cotangent to every position: the provider detects it on the
+    device, hands the region a stride-0 view, and gives the same Jacobians as with the detection off."""
+    from latent_bounded_interfaces_amd.backward import StructuredInterfacePullbackProvider
+
+    model = _model(device)
+    ids = torch.randint(0, 61, (2, 10), generator=torch.Generator().manual_seed(3)).to(device)
+    _, cache = model.forward_with_cache(ids)
+    seen = []
+    inner = model.region_backend.input_pullback_basis
+
+    def spy(*, cache, output_cotangent_basis):
+        seen.append(output_cotangent_basis.stride(2))
+        return inner(cache=cache, output_cotangent_basis=output_cotangent_basis)
+
+    model.region_backend.input_pullback_basis = spy
+    try:
+        results = {}
+        for mode in ("off", "verify", "verify_once"):
+            seen.clear()
+            provider = StructuredInterfacePullbackProvider(position_constant_update=mode)
+            results[mode] = provider.materialize_state_jacobian_t(model=model, cache=cache)
+            assert all(s != 0 for s in seen) if mode == "off" else all(s == 0 for s in seen), (mode, seen)
+            if mode == "verify_once":
+                assert provider._constant_over_positions == {type(model.interface): True}
+    finally:
+        del model.region_backend.input_pullback_basis
+    for mode in ("verify", "verify_once"):
+        for a, b in zip(results[mode], results["off"]):
+            assert float((a - b).abs().max()) <= 2e-6 * float(b.abs().max())
+    with pytest.raises(ValueError, match="position_constant_update"):
+        StructuredInterfacePullbackProvider(position_constant_update="maybe")
+
+
 @pytest.mark.parametrize("layers,per_region", [(6, 2), (4, 1), (2, 2)])
 def test_scan_backward_step_reproduces_dense_gradients(layers, per_region, device):
     from latent_bounded_interfaces_amd.backward import StructuredInterfacePullbackProvider, lbi_scan_backward_step

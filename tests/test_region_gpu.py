@@ -214,6 +214,56 @@ def test_region_pullback_fp32_matches_autograd(case, device):
     assert _max_rel(got.cpu(), want) <= 2e-5, _max_rel(got.cpu(), want)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kernels_take_position_constant_cotangents(dtype, device):
+    """[B,P,1,*] inputs (the same cotangent at every position) give exactly what their expanded copies give."""
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(5)
+    b, p, t, dim, hidden = 2, 3, 7, 40, 24
+    g = torch.randn(b, p, t, dim).to(dtype).to(device)
+    x = torch.randn(b, t, dim, device=device)
+    w = (1 + 0.1 * torch.randn(dim)).to(dtype).to(device)
+    res1 = torch.randn(b, p, 1, dim, device=device)
+    total, branch = region.rmsnorm_pullback(g, x, w, 1e-5, res1, want_branch=True)
+    want_total, want_branch = region.rmsnorm_pullback(g, x, w, 1e-5, res1.expand(b, p, t, dim).contiguous(),
+                                                      want_branch=True)
+    assert torch.equal(total, want_total) and torch.equal(branch, want_branch)
+    assert total.data_ptr() != res1.data_ptr()
+    gd1 = torch.randn(b, p, 1, hidden).to(dtype).to(device)
+    fc1 = (2 * torch.randn(b, t, 2 * hidden)).to(dtype).to(device)
+    got = region.gated_mlp_pullback(gd1, fc1)
+    assert torch.equal(got, region.gated_mlp_pullback(gd1.expand(b, p, t, hidden).contiguous(), fc1))
+    with pytest.raises(ValueError, match=r"\[B, P, 1, hidden\]"):
+        region.gated_mlp_pullback(gd1.expand(b, p, 2, hidden), fc1)
+    with pytest.raises(ValueError, match=r"\[B, P, 1, D\]"):
+        region.rmsnorm_pullback(g, x, w, 1e-5, torch.zeros(b, p, 2, dim, device=device), want_branch=False)
+
+
+@pytest.mark.parametrize("case", REGION_CASES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_region_pullback_of_an_expanded_view(case, dtype, device):
+    """A stride-0 basis over positions takes the shortened path through the last block; the result is that of
+    the dense copy of the same basis (up to the rounding of a product run on fewer rows)."""
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+
+    dim, heads, kv, hd, hidden, layers, d_conv, inter, b, p, t = case
+    backend = oreg.make_backend(dim=dim, n_heads=heads, n_kv_heads=kv, head_dim=hd, hidden=hidden, layers=layers,
+                                d_conv=d_conv, rope_interleaved=inter, rope_base=1000.0, seed=dim, dtype=dtype).to(device)
+    torch.manual_seed(t)
+    x = torch.randn(b, t, dim, device=device)
+    pooled = torch.randn(b, p, 1, dim, device=device)
+    with torch.no_grad():
+        _, cache = backend.forward_region(region_input=x, region_index=0)
+    lowering = HipTransformerLowering()
+    view = pooled.expand(b, p, t, dim)
+    assert view.stride(2) == 0
+    got = lowering.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=view)
+    want = lowering.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=view.contiguous())
+    assert got.shape == want.shape == (b, p, t, dim)
+    assert _max_rel(got.cpu(), want.cpu()) <= (1e-6 if dtype == torch.float32 else _tol(dtype))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("residual_in_fp32", [True, False])
 def test_region_pullback_16bit_matches_fp32_path(dtype, residual_in_fp32, device):
