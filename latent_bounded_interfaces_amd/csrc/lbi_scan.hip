@@ -15,6 +15,7 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include "lbi_scan_colsplit.h"
 #include "lbi_scan_split.h"
 
 namespace lbi {
@@ -487,7 +488,14 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
             // MFMA).  fp32 storage would need 9: measured 4 % faster than the fp32-MFMA kernel
             // and slightly less accurate (the part clocks down under dense bf16 MFMA load), so
             // it is opt-in: LBI_SCAN_SPLIT_FP32=1.
-            if constexpr (std::is_same<Tin, bf16_raw>::value) return scan_split::launch<Tin>(mats, out, g, cot, B, K, stream);
+            // Matrices only: the column-owner form (a wave keeps its 16 columns of the suffix in registers, no
+            // barrier between steps; 0.99 ms against 1.22 ms at B=64, K=128).  With the cotangent chain: the
+            // row-owner form, which carries the chain in its row dot products.  LBI_SCAN_ROW_OWNER=1 forces it.
+            if constexpr (std::is_same<Tin, bf16_raw>::value) {
+                static const bool row_owner = std::getenv("LBI_SCAN_ROW_OWNER") && std::atoi(std::getenv("LBI_SCAN_ROW_OWNER"));
+                if (!cot && !row_owner && K >= 1) return scan_col::launch(mats, out, B, K, stream);
+                return scan_split::launch<Tin>(mats, out, g, cot, B, K, stream);
+            }
             if constexpr (std::is_same<Tin, float>::value) {
                 static const bool split_fp32 =
                     std::getenv("LBI_SCAN_SPLIT_FP32") && std::atoi(std::getenv("LBI_SCAN_SPLIT_FP32"));

@@ -136,6 +136,28 @@ def test_fused_scan_and_cotangents(shape, dtype, device):
     assert float(((cot.cpu().double() - truth).abs() / scale).max()) <= 1e-5
 
 
+@pytest.mark.parametrize("shape", [(2, 5, 256), (9, 1, 256), (3, 12, 256), (2, 6, 64)])
+def test_fused_scan_and_cotangents_bf16_storage(shape, device):
+    """bf16 storage at d=256: the fused entry runs the row-owner split kernel (with the cotangent chain), the
+    matrices-only entry the column-owner one; both are exact-split fp32 products in different summation orders."""
+    from latent_bounded_interfaces_amd.hip.interface import (
+        suffix_scan_pullbacks,
+        suffix_scan_pullbacks_and_cotangents,
+    )
+
+    bsz, count, rank = shape
+    mats, g = oscan.make_scan_inputs(bsz, count, rank, kind="randn", seed=6)
+    mats = mats.to(torch.bfloat16)
+    mats_d, g_d = mats.to(device), g.to(device)
+    out, cot = suffix_scan_pullbacks_and_cotangents(mats_d, g_d)
+    truth = oscan.suffix_scan_sequential(mats.float(), dtype=torch.float64)
+    assert _rel_err(out.cpu(), truth) <= 1e-5
+    assert _rel_err(suffix_scan_pullbacks(mats_d).cpu(), truth) <= 1e-5
+    want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+    scale = want.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+    assert float(((cot.cpu().double() - want).abs() / scale).max()) <= 1e-5
+
+
 def test_benchmark_shape_properties(device):
     """B=64, K=128, d=256: size-independent checks (recurrence, identity tail, reruns bit-stable)."""
     from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents, suffix_scan_pullbacks
