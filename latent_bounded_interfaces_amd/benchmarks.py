@@ -57,14 +57,15 @@ class PullbackCall:
         self.out = tuple(torch.empty_like(g) for _ in range(3))
         need = int(self.lib.lbi_attn_pullback_workspace_bytes(self.B, self.H, self.T, self.Dh, self.P, self.dtype))
         self.ws = torch.empty(max(need, 256), device=q.device, dtype=torch.uint8)
-        self.stream = _lib.current_stream_ptr(q.device)
+        self.device = q.device
 
     def __call__(self):
         q, k, v, g = self.args
         st = self.lib.lbi_attn_pullback(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(),
                                         self.out[0].data_ptr(), self.out[1].data_ptr(), self.out[2].data_ptr(),
                                         self.ws.data_ptr(), self.ws.numel(), self.B, self.H, self.T, self.Dh, self.P,
-                                        self.scale, int(self.causal), self.dtype, self.stream)
+                                        self.scale, int(self.causal), self.dtype,
+                                        _lib.current_stream_ptr(self.device))
         _lib.check(st, "lbi_attn_pullback")
         return self.out
 
@@ -111,12 +112,31 @@ def measure(B, H, T, Dh, P, dtype, *, causal=True, warmup=3, iters=10, device="c
     }
 
 
+def graph_replay_ms(call, *, iters: int = 50) -> float:
+    """Median time of one replay of ``call`` captured into a HIP graph (the launch-bound small shapes:
+    one graph launch instead of one launch per kernel)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    median_ms, _, _, _ = time_call(graph.replay, warmup=5, iters=iters)
+    return median_ms
+
+
 def attention_section(steps: int = 5) -> dict:
     """The two attention configurations reported beside the scan headline."""
     out = {}
     out["attn_pullback_bf16_B4_H16_T4096_Dh128_P16"] = measure(4, 16, 4096, 128, 16, torch.bfloat16, iters=steps)
     torch.cuda.empty_cache()
-    out["attn_pullback_fp16_B8_H8_T128_Dh64_P4"] = measure(8, 8, 128, 64, 4, torch.float16, iters=max(steps, 20))
+    small = measure(8, 8, 128, 64, 4, torch.float16, iters=max(steps, 20))
+    q, k, v, g = make_inputs(8, 8, 128, 64, 4, torch.float16, "cuda")
+    small["graph_replay_ms"] = graph_replay_ms(PullbackCall(q, k, v, g, 1.0 / math.sqrt(64), True))
+    out["attn_pullback_fp16_B8_H8_T128_Dh64_P4"] = small
     return out
 
 
