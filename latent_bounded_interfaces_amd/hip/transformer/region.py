@@ -39,11 +39,12 @@ def _require_cuda(*tensors: torch.Tensor) -> None:
 
 
 def rmsnorm_pullback(g_out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
-                     g_residual: torch.Tensor | None, *, want_branch: bool) -> tuple[torch.Tensor, torch.Tensor | None]:
+                     g_residual: torch.Tensor | None, *, want_branch: bool,
+                     keep_residual: bool = False) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``g_out [B,P,T,D]`` through RMSNorm at input ``x [B,T,D]``, plus ``g_residual`` (fp32).
 
     Returns ``(sum fp32, sum in g_out.dtype or None)``.  ``g_residual [B,P,T,D]`` is overwritten with the
-    sum; ``g_residual [B,P,1,D]`` (the same cotangent at every position) is read only.
+    sum unless ``keep_residual``; ``g_residual [B,P,1,D]`` (the same cotangent at every position) is read only.
     """
     _require_cuda(g_out, x, weight)
     bsz, basis, seqlen, dim = g_out.shape
@@ -58,7 +59,7 @@ def rmsnorm_pullback(g_out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor,
         if g_residual.dtype != torch.float32 or not g_residual.is_contiguous():
             raise ValueError("rmsnorm_pullback: g_residual must be a contiguous fp32 tensor")
         if g_residual.shape == g_out.shape:
-            total = g_residual
+            total = torch.empty_like(g_residual) if keep_residual else g_residual
         elif g_residual.shape == (bsz, basis, 1, dim):
             total = torch.empty(g_out.shape, device=g_out.device, dtype=torch.float32)
             shared = 1
@@ -252,10 +253,11 @@ def _conv_grads(sink: dict, conv: Any, g_out: torch.Tensor, x_pre: torch.Tensor)
 
 
 def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor | None, g_residual: torch.Tensor,
-                          kernel_mode: str, want_branch: bool,
-                          param_grads: dict | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
+                          kernel_mode: str, want_branch: bool, param_grads: dict | None = None,
+                          keep_residual: bool = False) -> tuple[torch.Tensor, torch.Tensor | None]:
     """One block, backwards.  ``g_residual`` (fp32, [B,P,T,D]) is the cotangent of the block's
-    residual output and is updated in place (``[B,P,1,D]``: the same at every position, read only);
+    residual output and is updated in place (``[B,P,1,D]``: the same at every position, read only; with
+    ``keep_residual`` a full-size one is left untouched too);
     ``g_hidden`` is the cotangent of its hidden output
     in the weight dtype (``None``: equal to ``g_residual``).  Returns the cotangent of
     ``hidden (+ residual)`` at the block input in fp32 and, if ``want_branch``, also rounded to
@@ -284,7 +286,7 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
         _norm_weight_grad(param_grads, block.norm2, g_norm2, m_cache.norm_input)
     # res2 feeds norm2 and the residual output
     g_res2, g_attn_out = rmsnorm_pullback(g_norm2, m_cache.norm_input, block.norm2.weight, block.norm2.eps,
-                                          g_residual, want_branch=True)
+                                          g_residual, want_branch=True, keep_residual=keep_residual)
     del g_norm2
 
     # attention: res2 = out_proj(heads) + res1
@@ -335,7 +337,10 @@ def _pull_back_region(backend: Any, cache: Any, cotangent: torch.Tensor, kernel_
         # block's down-projection product then runs on one row per (b, p) and the kernels read [B,P,1,*].
         g = cotangent[:, :, :1].to(device=device, dtype=torch.float32, copy=True).contiguous()
     else:
-        g = cotangent.to(device=device, dtype=torch.float32, copy=True).contiguous()
+        g = cotangent.to(device=device, dtype=torch.float32).contiguous()
+    # the caller's tensor itself when it already is fp32, contiguous and on the device: the last block then
+    # writes its residual sum to a new tensor instead of updating in place
+    borrowed = g.data_ptr() == cotangent.data_ptr()
     g_branch = None
     for offset in range(end - start - 1, -1, -1):
         layer_cache = cache.layer_caches[offset]
@@ -343,7 +348,8 @@ def _pull_back_region(backend: Any, cache: Any, cotangent: torch.Tensor, kernel_
         # hidden and residual at a block input enter only through their sum, so one cotangent
         # (fp32, and its rounded copy for the first product of the block before) is carried
         g, g_branch = _layer_input_pullback(block, layer_cache, g_branch, g, kernel_mode, want_branch=offset > 0,
-                                            param_grads=param_grads)
+                                            param_grads=param_grads, keep_residual=borrowed)
+        borrowed = False
     return g
 
 

@@ -208,10 +208,12 @@ def test_region_pullback_fp32_matches_autograd(case, device):
     gpu_backend = backend.to(device)
     with torch.no_grad():
         _, cache = gpu_backend.forward_region(region_input=x.to(device), region_index=0)
+    basis_d = basis.to(device)
     got = HipTransformerLowering().input_pullback_basis(backend=gpu_backend, cache=cache,
-                                                        output_cotangent_basis=basis.to(device))
+                                                        output_cotangent_basis=basis_d)
     assert got.shape == basis.shape and got.dtype == basis.dtype and got.is_cuda
     assert _max_rel(got.cpu(), want) <= 2e-5, _max_rel(got.cpu(), want)
+    assert torch.equal(basis_d.cpu(), basis) and got.data_ptr() != basis_d.data_ptr()  # the caller's tensor is read only
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
