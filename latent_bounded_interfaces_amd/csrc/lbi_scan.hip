@@ -483,23 +483,27 @@ template <typename Tin>
 int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, int K, int d, hipStream_t stream) {
     switch (d) {
         case 256: {
-            // bf16 storage runs on the 16-bit matrix pipes with exact three-way splits of the
-            // running suffix (3 bf16 products per fp32 product instead of one 16x slower fp32
-            // MFMA).  fp32 storage would need 9: measured 4 % faster than the fp32-MFMA kernel
-            // and slightly less accurate (the part clocks down under dense bf16 MFMA load), so
-            // it is opt-in: LBI_SCAN_SPLIT_FP32=1.
-            // Matrices only: the column-owner form (a wave keeps its 16 columns of the suffix in registers, no
-            // barrier between steps; 0.99 ms against 1.22 ms at B=64, K=128).  With the cotangent chain: the
-            // row-owner form, which carries the chain in its row dot products.  LBI_SCAN_ROW_OWNER=1 forces it.
+            // bf16 storage runs on the 16-bit matrix pipes: the running suffix enters each product as bf16
+            // planes (hi + mid + lo), the bf16 matrix as it is, accumulation in fp32.  Three planes (the default)
+            // are the fp32 value exactly.  LBI_SCAN_BF16_PLANES=2 rounds that operand to 16 significand bits,
+            // 256 times finer than the bf16 rounding of the inputs themselves (error against fp64 <= 2e-4 at
+            // K=128 where 2e-2 is asked of 16-bit storage), for two thirds of the products: 10-13 % faster.
+            // Matrices only: the column-owner kernel (a wave keeps its 16 columns of the suffix in registers, no
+            // barrier between steps).  With the cotangent chain: the row-owner kernel, whose row dot products
+            // carry the chain.  LBI_SCAN_ROW_OWNER=1 forces the latter.
+            // fp32 storage would need 3 x 3 planes: measured 4 % faster than the fp32-MFMA kernel and slightly
+            // less accurate (the part clocks down under dense bf16 MFMA load), so it is opt-in:
+            // LBI_SCAN_SPLIT_FP32=1.
             if constexpr (std::is_same<Tin, bf16_raw>::value) {
                 static const bool row_owner = std::getenv("LBI_SCAN_ROW_OWNER") && std::atoi(std::getenv("LBI_SCAN_ROW_OWNER"));
-                if (!cot && !row_owner && K >= 1) return scan_col::launch(mats, out, B, K, stream);
-                return scan_split::launch<Tin>(mats, out, g, cot, B, K, stream);
+                static const int planes = std::getenv("LBI_SCAN_BF16_PLANES") ? std::atoi(std::getenv("LBI_SCAN_BF16_PLANES")) : 3;
+                if (!cot && !row_owner && K >= 1) return scan_col::launch(mats, out, B, K, planes, stream);
+                return scan_split::launch<Tin>(mats, out, g, cot, B, K, planes, stream);
             }
             if constexpr (std::is_same<Tin, float>::value) {
                 static const bool split_fp32 =
                     std::getenv("LBI_SCAN_SPLIT_FP32") && std::atoi(std::getenv("LBI_SCAN_SPLIT_FP32"));
-                if (split_fp32) return scan_split::launch<Tin>(mats, out, g, cot, B, K, stream);
+                if (split_fp32) return scan_split::launch<Tin>(mats, out, g, cot, B, K, 3, stream);
             }
             return launch_mfma<Tin, 256, 32, 64>(mats, out, g, cot, B, K, stream);
         }

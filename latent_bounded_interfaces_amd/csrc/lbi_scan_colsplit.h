@@ -60,11 +60,20 @@ __device__ __forceinline__ void split2(float x0, float x1, unsigned& hi, unsigne
     lo = pack_bf16(r0 - bf16_lo(mid), r1 - bf16_hi(mid));
 }
 
+// hi and mid only: x rounded to 16 significand bits
+__device__ __forceinline__ void split2_top(float x0, float x1, unsigned& hi, unsigned& mid) {
+    hi = pack_bf16(x0, x1);
+    mid = pack_bf16(x0 - bf16_lo(hi), x1 - bf16_hi(hi));
+}
+
 __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0,
                                                    0);
 }
 
+// NP = planes of the running suffix that enter the products: 3 is exact (the fp32 value), 2 rounds the operand to
+// 16 significand bits (hi + mid); the accumulation and the stored result are fp32 either way.
+template <int NP>
 __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __restrict__ mats, float* __restrict__ out,
                                                           int B, int K) {
     extern __shared__ __align__(16) char smem[];
@@ -100,9 +109,9 @@ __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __res
     };
 
     f32x4 acc[MT];
-    u32x4 bfr[KS][3];      // B fragments of the current step: [k-step][plane]
-    u32x4 late[2][3];      // fragments of the last two k-steps of the next step, until this step is done with its own
-    u32x2 even_words[3];   // packed planes of the even tile of a pair, waiting for the odd one
+    u32x4 bfr[KS][NP];      // B fragments of the current step: [k-step][plane]
+    u32x4 late[2][NP];      // fragments of the last two k-steps of the next step, until this step is done with its own
+    u32x2 even_words[NP];   // packed planes of the even tile of a pair, waiting for the odd one
 
     // Row tile mt of step r is complete in acc: store it, split it, and with its pair partner form the B fragments of
     // k-step mt / 2 of the next step.  Accumulator layout: lane (n, g), register e <-> row 16 mt + 4 g + e; fragment
@@ -114,16 +123,21 @@ __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __res
 #pragma unroll
         for (int e = 0; e < 4; ++e) o_r[(size_t)e * D] = tot[e];
         unsigned w[3][2];
-        split2(tot[0], tot[1], w[0][0], w[1][0], w[2][0]);
-        split2(tot[2], tot[3], w[0][1], w[1][1], w[2][1]);
+        if (NP == 3) {
+            split2(tot[0], tot[1], w[0][0], w[1][0], w[2][0]);
+            split2(tot[2], tot[3], w[0][1], w[1][1], w[2][1]);
+        } else {
+            split2_top(tot[0], tot[1], w[0][0], w[1][0]);
+            split2_top(tot[2], tot[3], w[0][1], w[1][1]);
+        }
         if ((mt & 1) == 0) {
 #pragma unroll
-            for (int p = 0; p < 3; ++p) even_words[p] = u32x2{w[p][0], w[p][1]};
+            for (int p = 0; p < NP; ++p) even_words[p] = u32x2{w[p][0], w[p][1]};
             return;
         }
         const int ks = mt >> 1;
 #pragma unroll
-        for (int p = 0; p < 3; ++p) {
+        for (int p = 0; p < NP; ++p) {
             u32x4 frag;
 #pragma unroll
             for (int hw = 0; hw < 2; ++hw) {
@@ -191,11 +205,10 @@ __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __res
                     for (int t = 0; t < 4; ++t)
                         a[t] = *reinterpret_cast<const u32x4*>(stage + (mt + t) * 16 * CHUNK_ROW_BYTES + frag_off[s]);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[mt + t] = mma(a[t], bfr[ks][2], first ? zero : acc[mt + t]);
+                    for (int p = NP - 1; p >= 0; --p)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[mt + t] = mma(a[t], bfr[ks][1], acc[mt + t]);
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[mt + t] = mma(a[t], bfr[ks][0], acc[mt + t]);
+                        for (int t = 0; t < 4; ++t)
+                            acc[mt + t] = mma(a[t], bfr[ks][p], (first && p == NP - 1) ? zero : acc[mt + t]);
                     if (c == NCHUNK - 1 && s == CHUNK_KS - 1) {
 #pragma unroll
                         for (int t = 0; t < 4; ++t) finish_tile(mt + t, r, true);
@@ -206,13 +219,14 @@ __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __res
 #pragma unroll
         for (int s = 0; s < CHUNK_KS; ++s)
 #pragma unroll
-            for (int p = 0; p < 3; ++p) bfr[KS - CHUNK_KS + s][p] = late[s][p];
+            for (int p = 0; p < NP; ++p) bfr[KS - CHUNK_KS + s][p] = late[s][p];
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 }
 
-inline int launch(const void* mats, void* out, int B, int K, hipStream_t stream) {
-    auto kern = scan_colsplit_kernel;
+template <int NP>
+int launch_planes(const void* mats, void* out, int B, int K, hipStream_t stream) {
+    auto kern = scan_colsplit_kernel<NP>;
     static bool attr_done[16] = {};
     int dev = 0;
     LBI_HIP_CHECK(hipGetDevice(&dev));
@@ -226,6 +240,10 @@ inline int launch(const void* mats, void* out, int B, int K, hipStream_t stream)
                        static_cast<float*>(out), B, K);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
+}
+
+inline int launch(const void* mats, void* out, int B, int K, int planes, hipStream_t stream) {
+    return planes >= 3 ? launch_planes<3>(mats, out, B, K, stream) : launch_planes<2>(mats, out, B, K, stream);
 }
 
 }  // namespace scan_col

@@ -71,7 +71,9 @@ template <> struct Chunk<float> {
     static constexpr int K_PER_CHUNK = 32, K_PER_LANE = 16, T_STEPS = 2, NA = 3;
 };
 
-template <typename Tin, bool COT>
+// NP = planes of the running suffix that enter the products: 3 is exact; 2 (bf16 storage only) rounds that operand
+// to 16 significand bits (hi + mid), accumulation and stored results stay fp32.
+template <typename Tin, bool COT, int NP>
 __global__ __launch_bounds__(NT) void scan_split_kernel(const Tin* __restrict__ mats, float* __restrict__ out,
                                                         const float* __restrict__ g, float* __restrict__ cot, int B,
                                                         int K) {
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(NT) void scan_split_kernel(const Tin* __restrict__ 
 
     extern __shared__ __align__(16) char smem[];
     unsigned short* planes = reinterpret_cast<unsigned short*>(smem);        // [3][CB][PITCH]
-    float* vbuf = reinterpret_cast<float*>(smem + PLANES_BYTES);              // (COT) [2][D]
+    float* vbuf = reinterpret_cast<float*>(smem + (size_t)NP * PLANE * 2);  // (COT) [2][D], behind the NP planes
 
     const int id = blockIdx.x;
     const int slot_id = id >> 3;
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(NT) void scan_split_kernel(const Tin* __restrict__ 
             split2(val, 0.0f, hi, mid, lo);
             planes[0 * PLANE + col * PITCH + row] = (unsigned short)hi;
             planes[1 * PLANE + col * PITCH + row] = (unsigned short)mid;
-            planes[2 * PLANE + col * PITCH + row] = (unsigned short)lo;
+            if (NP > 2) planes[2 * PLANE + col * PITCH + row] = (unsigned short)lo;
         }
         if (COT) {
             const float* g_b = g + (size_t)b * D;
@@ -152,10 +154,10 @@ __global__ __launch_bounds__(NT) void scan_split_kernel(const Tin* __restrict__ 
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[o][j][e] = 0.0f;
         float vdot = 0.0f;
-        u32x4 bfr[2][3][2];
-        auto load_b = [&](u32x4 (&dst)[3][2], int k_off) {
+        u32x4 bfr[2][NP][2];
+        auto load_b = [&](u32x4 (&dst)[NP][2], int k_off) {
 #pragma unroll
-            for (int sp = 0; sp < 3; ++sp) {
+            for (int sp = 0; sp < NP; ++sp) {
                 const char* bp = smem + (size_t)sp * PLANE * 2 + b_lane + k_off * 2;
                 dst[sp][0] = *reinterpret_cast<const u32x4*>(bp);
                 dst[sp][1] = *reinterpret_cast<const u32x4*>(bp + 32 * PITCH * 2);
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(NT) void scan_split_kernel(const Tin* __restrict__ 
                     load_b(bfr[slot_b ^ 1], kc_n * C::K_PER_CHUNK + 8 * t_n);
                 }
 #pragma unroll
-                for (int sp = 2; sp >= 0; --sp)  // small planes first
+                for (int sp = NP - 1; sp >= 0; --sp)  // small planes first
 #pragma unroll
                     for (int ap = NA - 1; ap >= 0; --ap) {
                         if (ap + sp > LBI_SPLIT_MAX_ORDER) continue;
@@ -255,7 +257,7 @@ __global__ __launch_bounds__(NT) void scan_split_kernel(const Tin* __restrict__ 
                 unsigned short* dst = planes + col * PITCH + row;
                 *reinterpret_cast<u32x2*>(dst) = u32x2{hi0, hi1};
                 *reinterpret_cast<u32x2*>(dst + PLANE) = u32x2{mid0, mid1};
-                *reinterpret_cast<u32x2*>(dst + 2 * PLANE) = u32x2{lo0, lo1};
+                if (NP > 2) *reinterpret_cast<u32x2*>(dst + 2 * PLANE) = u32x2{lo0, lo1};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o_r[(size_t)(row + e) * D + c0 + col] = tot[e];
             }
@@ -271,18 +273,18 @@ __global__ __launch_bounds__(NT) void scan_split_kernel(const Tin* __restrict__ 
     }
 }
 
-template <typename Tin>
-int launch(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
-    const size_t lds_bytes = PLANES_BYTES + (cot ? 2 * D * sizeof(float) : 0);
+template <typename Tin, int NP>
+int launch_planes(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
+    const size_t lds_bytes = (size_t)NP * PLANE * 2 + (cot ? 2 * D * sizeof(float) : 0);
     const dim3 grid(((B + 7) / 8) * 8 * NB);
     if (cot) {
-        auto kern = scan_split_kernel<Tin, true>;
+        auto kern = scan_split_kernel<Tin, true, NP>;
         LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds_bytes));
         hipLaunchKernelGGL(kern, grid, dim3(NT), lds_bytes, stream, static_cast<const Tin*>(mats),
                            static_cast<float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), B, K);
     } else {
-        auto kern = scan_split_kernel<Tin, false>;
+        auto kern = scan_split_kernel<Tin, false, NP>;
         LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)lds_bytes));
         hipLaunchKernelGGL(kern, grid, dim3(NT), lds_bytes, stream, static_cast<const Tin*>(mats),
@@ -291,6 +293,13 @@ int launch(const void* mats, void* out, const void* g, void* cot, int B, int K, 
     }
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
+}
+
+// planes: 3 = exact; 2 = 16-bit suffix operand, bf16 storage only (fp32 storage always runs exact).
+template <typename Tin>
+int launch(const void* mats, void* out, const void* g, void* cot, int B, int K, int planes, hipStream_t stream) {
+    if (planes < 3 && Chunk<Tin>::NA == 1) return launch_planes<Tin, 2>(mats, out, g, cot, B, K, stream);
+    return launch_planes<Tin, 3>(mats, out, g, cot, B, K, stream);
 }
 
 }  // namespace scan_split

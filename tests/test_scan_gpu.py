@@ -23,6 +23,12 @@ SHAPES = [
 ]
 
 
+# bf16 storage at d=256 runs exact three-plane products by default and meets the fp32 bar; the opt-in two-plane
+# form (LBI_SCAN_BF16_PLANES=2, tested in a subprocess below) rounds the suffix operand to 16 significand bits.
+BF16_D256_BAR = 1e-5
+BF16_D256_TWO_PLANE_BAR = 2e-4
+
+
 def _rel_err(actual: torch.Tensor, truth: torch.Tensor) -> float:
     """max over suffix matrices of max|diff| / max|truth| (fp64 truth)."""
     diff = (actual.double() - truth).abs().flatten(2).max(dim=2).values
@@ -76,7 +82,8 @@ def test_low_precision_storage_promotes_to_fp32(shape, dtype, device):
     assert out.dtype == torch.float32
     truth = oscan.suffix_scan_sequential(mats.float(), dtype=torch.float64)
     # Inputs are rounded before both sides see them, so only fp32 accumulation differs.
-    assert _rel_err(out, truth) <= 1e-5
+    bar = BF16_D256_BAR if (dtype == torch.bfloat16 and rank == 256) else 1e-5
+    assert _rel_err(out, truth) <= bar
     assert torch.allclose(out, oscan.suffix_scan_sequential(mats.float()), atol=2e-1, rtol=5e-3)
 
 
@@ -151,8 +158,9 @@ def test_fused_scan_and_cotangents_bf16_storage(shape, device):
     mats_d, g_d = mats.to(device), g.to(device)
     out, cot = suffix_scan_pullbacks_and_cotangents(mats_d, g_d)
     truth = oscan.suffix_scan_sequential(mats.float(), dtype=torch.float64)
-    assert _rel_err(out.cpu(), truth) <= 1e-5
-    assert _rel_err(suffix_scan_pullbacks(mats_d).cpu(), truth) <= 1e-5
+    bar = BF16_D256_BAR if rank == 256 else 1e-5
+    assert _rel_err(out.cpu(), truth) <= bar
+    assert _rel_err(suffix_scan_pullbacks(mats_d).cpu(), truth) <= bar
     want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
     scale = want.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
     assert float(((cot.cpu().double() - want).abs() / scale).max()) <= 1e-5
@@ -198,7 +206,7 @@ def test_benchmark_shape_properties(device):
     rel = (out_bf16 - out_ref).abs().flatten(2).amax(dim=2) / out_ref.abs().flatten(2).amax(dim=2)
     assert float(rel.max()) <= 2e-2
     truth_bf = oscan.suffix_scan_sequential(mats_bf16[pick].float().cpu(), dtype=torch.float64)
-    assert _rel_err(out_bf16[pick].cpu(), truth_bf) <= 1e-5
+    assert _rel_err(out_bf16[pick].cpu(), truth_bf) <= BF16_D256_BAR
 
 
 def test_backward_module_contract(device):
@@ -254,5 +262,31 @@ def test_split_fp32_variant_in_subprocess(device):
         "print(e, ec); sys.exit(0 if e <= 1e-5 and ec <= 1e-5 else 1)"
     ) % str(Path(__file__).resolve().parents[1])
     env = dict(os.environ, LBI_SCAN_SPLIT_FP32="1")
+    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stdout + res.stderr
+
+
+def test_two_plane_bf16_mode_in_subprocess(device):
+    """LBI_SCAN_BF16_PLANES=2: the suffix operand rounded to 16 significand bits stays a hundred times inside the
+    2e-2 asked of 16-bit storage, in the column-owner kernel (matrices only) and the row-owner kernel (with the
+    cotangent chain), at K=128 too."""
+    import os
+    import subprocess
+    import sys
+
+    code = (
+        "import torch, sys; sys.path.insert(0, %r);"
+        "from oracle import scan as o;"
+        "from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks as s, "
+        "suffix_scan_pullbacks_and_cotangents as f;"
+        "worst = 0.0\n"
+        "for shape, kind in (((3, 9, 256), 'randn'), ((2, 128, 256), 'near_identity')):\n"
+        "    m, g = o.make_scan_inputs(*shape, kind=kind, seed=5); m = m.to(torch.bfloat16)\n"
+        "    t = o.suffix_scan_sequential(m.float(), dtype=torch.float64)\n"
+        "    for out in (s(m.cuda()), f(m.cuda(), g.cuda())[0]):\n"
+        "        worst = max(worst, float(((out.cpu().double() - t).abs().flatten(2).amax(2) / t.abs().flatten(2).amax(2)).max()))\n"
+        "print(worst); sys.exit(0 if 1e-7 < worst <= %g else 1)"
+    ) % (str(Path(__file__).resolve().parents[1]), BF16_D256_TWO_PLANE_BAR)
+    env = dict(os.environ, LBI_SCAN_BF16_PLANES="2")
     res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert res.returncode == 0, res.stdout + res.stderr
