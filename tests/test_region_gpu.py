@@ -366,3 +366,37 @@ def test_parameter_vjp_16bit_matches_fp32_path(dtype, device):
     for name, w in want.items():
         assert got[name].dtype == dtype
         assert _max_rel(got[name].cpu(), w) <= 3e-2, (name, _max_rel(got[name].cpu(), w))
+
+
+def test_kernels_at_the_end_to_end_scale(device):
+    """B=8, P=64, T=1024, d_model 768 / hidden 3072 (up to 3.2e9 elements per tensor, past 2^31): the last batch
+    element and direction of every kernel's output equal the same kernel run on that slice alone."""
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(0)
+    b, p, t, heads, hd, dim, hidden = 8, 64, 1024, 12, 64, 768, 3072
+    dt = torch.bfloat16
+    gd = torch.randn(b, p, t, hidden, device=device, dtype=dt)
+    fc1 = torch.randn(b, t, 2 * hidden, device=device, dtype=dt)
+    full = region.gated_mlp_pullback(gd, fc1)
+    assert torch.equal(full[-1, -1], region.gated_mlp_pullback(gd[-1:, -1:].contiguous(), fc1[-1:])[0, 0])
+    del gd, fc1, full
+    x = torch.randn(b, t, dim, device=device)
+    wn = (1 + 0.1 * torch.randn(dim, device=device)).to(dt)
+    gy = torch.randn(b, p, t, dim, device=device, dtype=dt)
+    res = torch.randn(b, p, t, dim, device=device)
+    tot, br = region.rmsnorm_pullback(gy, x, wn, 1e-5, res.clone(), want_branch=True)
+    tot1, br1 = region.rmsnorm_pullback(gy[-1:, -1:].contiguous(), x[-1:], wn, 1e-5, res[-1:, -1:].contiguous(),
+                                        want_branch=True)
+    assert torch.equal(tot[-1, -1], tot1[0, 0]) and torch.equal(br[-1, -1], br1[0, 0])
+    hs = region.attn_heads_split(gy, heads, hd)
+    assert torch.equal(hs[-1, -1], gy[-1, -1].view(t, heads, hd).transpose(0, 1))
+    del tot, br, res, hs, gy
+    dq, dk, dv = (torch.randn(b, p, heads, t, hd, device=device, dtype=dt) for _ in range(3))
+    w = torch.randn(3 * heads * hd, 1, 4, device=device, dtype=dt)
+    kw = dict(n_kv_heads=heads, rope_base=10000.0, rope_interleaved=False)
+    full = region.attn_qkv_conv_pullback(dq, dk, dv, w, **kw)
+    part = region.attn_qkv_conv_pullback(*(z[-1:, -1:].contiguous() for z in (dq, dk, dv)), w, **kw)
+    assert torch.equal(full[-1, -1], part[0, 0])
+    two = region.causal_conv1d_pullback(region.attn_qkv_pullback(dq, dk, dv, **kw), w)
+    assert int((two != full).sum()) <= full.numel() // 2000
