@@ -29,6 +29,10 @@ _MODE_BASIS_LIMIT = {
 }
 
 
+# sequence-length granularity of the matrix-core kernels (the generic kernels take any length)
+_MFMA_SEQ_MULTIPLE = 64
+
+
 def _validate(q, k, v, output_cotangent_basis) -> None:
     # reference cuda/transformer/__init__.py:21-26
     if q.dim() != 4 or k.shape != q.shape or v.shape != q.shape:
@@ -76,6 +80,16 @@ def attention_input_pullback_basis(
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     d_out = output_cotangent_basis.contiguous()
     bsz, heads, seqlen, head_dim = q.shape
+    if (causal and seqlen % _MFMA_SEQ_MULTIPLE and seqlen > _MFMA_SEQ_MULTIPLE // 2 and head_dim in (64, 128)
+            and q.dtype in (torch.float16, torch.bfloat16) and d_out.numel()):
+        # The matrix-core kernels take sequence lengths that are multiples of 64.  Under the causal mask, rows
+        # appended after the sequence change nothing before them: appended keys are masked for every real query,
+        # and appended queries carry a zero cotangent, so they add nothing to dK or dV.  Pad, run, cut.
+        pad = _MFMA_SEQ_MULTIPLE - seqlen % _MFMA_SEQ_MULTIPLE
+        padded = [torch.nn.functional.pad(t, (0, 0, 0, pad)) for t in (q, k, v, d_out)]
+        outs = attention_input_pullback_basis(*padded, softmax_scale=softmax_scale, causal=True, use_cuda=use_cuda,
+                                              kernel_mode="hip")
+        return tuple(o[..., :seqlen, :].contiguous() for o in outs)
     dq = torch.empty_like(d_out)
     dk = torch.empty_like(d_out)
     dv = torch.empty_like(d_out)

@@ -75,6 +75,8 @@ LOWP_CASES = [
     (121, (1, 2, 16, 64), 1), (129, (1, 2, 16, 64), 4), (11, (2, 2, 64, 64), 2), (12, (1, 3, 128, 128), 3),
     (13, (2, 1, 192, 64), 5), (14, (1, 2, 320, 128), 2), (15, (1, 1, 576, 128), 1), (16, (8, 8, 128, 64), 4),
     (17, (1, 2, 96, 64), 2), (18, (1, 1, 64, 32), 2), (19, (1, 2, 256, 64), 9), (20, (1, 1, 448, 64), 16),
+    # lengths that are no multiple of 64: causal calls are padded onto the matrix-core kernels
+    (21, (2, 2, 100, 64), 3), (22, (1, 1, 1000, 128), 2), (23, (1, 2, 33, 64), 2),
 ]
 
 
