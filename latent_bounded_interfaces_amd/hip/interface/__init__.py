@@ -29,9 +29,29 @@ def _validate(mats: torch.Tensor) -> tuple[int, int, int]:
     return bsz, count, rank
 
 
+#: interface widths the matrix-core scan kernels are built for
+_MFMA_WIDTHS = (32, 64, 128, 256)
+
+
+def _padded_width(rank: int) -> int:
+    """The matrix-core width a scan of ``rank x rank`` matrices is padded to, or ``rank`` itself when it is one
+    already, too small to matter (<= 16) or beyond the largest."""
+    if rank <= 16 or rank in _MFMA_WIDTHS:
+        return rank
+    return next((w for w in _MFMA_WIDTHS if w > rank), rank)
+
+
 def suffix_scan_pullbacks(mats: torch.Tensor) -> torch.Tensor:
     """``out[:, r] = mats[:, r] @ ... @ mats[:, K-1]``, ``out[:, K] = I``; fp32, input untouched."""
     bsz, count, rank = _validate(mats)
+    width = _padded_width(rank)
+    if width != rank and mats.numel():
+        # Products of zero-padded matrices are the zero-padded products, and the identity tail cuts to the
+        # identity: run the matrix-core kernel of the next width instead of the scalar kernel (several times
+        # faster even with the extra bytes).
+        pad = width - rank
+        wide = suffix_scan_pullbacks(torch.nn.functional.pad(mats, (0, pad, 0, pad)))
+        return wide[:, :, :rank, :rank].contiguous()
     mats = mats.contiguous()
     out = torch.empty((bsz, count + 1, rank, rank), device=mats.device, dtype=torch.float32)
     if out.numel() == 0:
@@ -76,6 +96,12 @@ def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor) ->
     bsz, count, rank = _validate(mats)
     if g.dim() != 2 or g.shape[0] != bsz or g.shape[1] != rank:
         raise ValueError("g must have shape [B, R]")
+    width = _padded_width(rank)
+    if width != rank and mats.numel():
+        pad = width - rank  # see suffix_scan_pullbacks; a zero-padded g leaves the first `rank` cotangents unchanged
+        wide, wide_cot = suffix_scan_pullbacks_and_cotangents(torch.nn.functional.pad(mats, (0, pad, 0, pad)),
+                                                              torch.nn.functional.pad(g, (0, pad)))
+        return wide[:, :, :rank, :rank].contiguous(), wide_cot[:, :, :rank].contiguous()
     mats = mats.contiguous()
     g32 = g.to(device=mats.device, dtype=torch.float32).contiguous()
     out = torch.empty((bsz, count + 1, rank, rank), device=mats.device, dtype=torch.float32)

@@ -19,6 +19,7 @@ SHAPES = [
     (1, 0, 1), (1, 1, 1), (1, 1, 4), (2, 3, 5), (2, 4, 8), (4, 8, 16), (1, 16, 64),
     (1, 2, 16), (2, 4, 32), (2, 8, 64), (1, 16, 128), (1, 8, 256),
     (4, 8, 32), (3, 5, 32), (9, 7, 64), (5, 3, 128), (3, 5, 256), (2, 6, 48), (2, 3, 33), (1, 4, 100),
+    (1, 3, 300), (2, 5, 12),  # widths the scalar kernel still runs: past the largest matrix-core width, and tiny
     (17, 2, 256), (1, 1, 256), (2, 0, 32),
 ]
 
