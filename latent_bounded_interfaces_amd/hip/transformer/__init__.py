@@ -29,8 +29,9 @@ _MODE_BASIS_LIMIT = {
 }
 
 
-# sequence-length granularity of the matrix-core kernels (the generic kernels take any length)
+# what the matrix-core kernels take (the generic kernels take any length and head dim up to 256)
 _MFMA_SEQ_MULTIPLE = 64
+_MFMA_HEAD_DIMS = (64, 128)
 
 
 def _validate(q, k, v, output_cotangent_basis) -> None:
@@ -80,16 +81,23 @@ def attention_input_pullback_basis(
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     d_out = output_cotangent_basis.contiguous()
     bsz, heads, seqlen, head_dim = q.shape
-    if (causal and seqlen % _MFMA_SEQ_MULTIPLE and seqlen > _MFMA_SEQ_MULTIPLE // 2 and head_dim in (64, 128)
-            and q.dtype in (torch.float16, torch.bfloat16) and d_out.numel()):
-        # The matrix-core kernels take sequence lengths that are multiples of 64.  Under the causal mask, rows
-        # appended after the sequence change nothing before them: appended keys are masked for every real query,
-        # and appended queries carry a zero cotangent, so they add nothing to dK or dV.  Pad, run, cut.
-        pad = _MFMA_SEQ_MULTIPLE - seqlen % _MFMA_SEQ_MULTIPLE
-        padded = [torch.nn.functional.pad(t, (0, 0, 0, pad)) for t in (q, k, v, d_out)]
-        outs = attention_input_pullback_basis(*padded, softmax_scale=softmax_scale, causal=True, use_cuda=use_cuda,
-                                              kernel_mode="hip")
-        return tuple(o[..., :seqlen, :].contiguous() for o in outs)
+    if q.dtype in (torch.float16, torch.bfloat16) and d_out.numel() and seqlen > _MFMA_SEQ_MULTIPLE // 2:
+        # The matrix-core kernels take head dims 64 and 128 and sequence lengths that are multiples of 64; everything
+        # else runs on the generic kernels, at a small fraction of their speed.  Two paddings are exact:
+        # * zero columns appended to the head dim add nothing to any dot product (the scale is passed explicitly)
+        #   and receive zero cotangents;
+        # * under the causal mask, zero rows appended after the sequence are invisible to every real query, and as
+        #   queries they carry a zero cotangent, so they add nothing to dK or dV.
+        wide_dim = next((w for w in _MFMA_HEAD_DIMS if w >= head_dim), head_dim)
+        ragged = seqlen % _MFMA_SEQ_MULTIPLE != 0
+        long_seq = seqlen + (_MFMA_SEQ_MULTIPLE - seqlen % _MFMA_SEQ_MULTIPLE) if (ragged and causal) else seqlen
+        if (wide_dim != head_dim or long_seq != seqlen) and long_seq % _MFMA_SEQ_MULTIPLE == 0 \
+                and wide_dim in _MFMA_HEAD_DIMS:
+            pads = (0, wide_dim - head_dim, 0, long_seq - seqlen)
+            padded = [torch.nn.functional.pad(t, pads) for t in (q, k, v, d_out)]
+            outs = attention_input_pullback_basis(*padded, softmax_scale=softmax_scale, causal=causal,
+                                                  use_cuda=use_cuda, kernel_mode="hip")
+            return tuple(o[..., :seqlen, :head_dim].contiguous() for o in outs)
     dq = torch.empty_like(d_out)
     dk = torch.empty_like(d_out)
     dv = torch.empty_like(d_out)

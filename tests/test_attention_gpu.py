@@ -77,6 +77,9 @@ LOWP_CASES = [
     (17, (1, 2, 96, 64), 2), (18, (1, 1, 64, 32), 2), (19, (1, 2, 256, 64), 9), (20, (1, 1, 448, 64), 16),
     # lengths that are no multiple of 64: causal calls are padded onto the matrix-core kernels
     (21, (2, 2, 100, 64), 3), (22, (1, 1, 1000, 128), 2), (23, (1, 2, 33, 64), 2),
+    # head dims below 128 that are not 64: zero-padded onto the matrix-core kernels (with the length, if causal)
+    (24, (1, 2, 128, 32), 3), (25, (2, 1, 192, 96), 2), (26, (1, 2, 70, 80), 2), (27, (1, 1, 64, 8), 1),
+    (28, (1, 1, 128, 160), 2),  # past 128: generic kernels
 ]
 
 
