@@ -249,12 +249,12 @@ template <int DH, int PB> constexpr size_t dq_ring_lds_bytes() {
     return 2 * (2 * 32 * DH * 2) + 4 * PB * 32 * DH * 2;  // K/V ring + d_out tiles of four waves
 }
 
-// PB is the direction block of the caller's choice for head dim 64 (4 or 8); head dim 128 has
+// PB is the direction block of the caller's choice (1, 2, 4, and 8 for head dim 64); head dim 128 has
 // accumulation registers for four.
 template <typename T, int DH, int PB, bool CAUSAL>
 void launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
                int H, int P, int T_len, float scale, hipStream_t stream) {
-    constexpr int PBK = DH == 128 ? 4 : PB;
+    constexpr int PBK = (DH == 128 && PB > 4) ? 4 : PB;
     const int n_qb = (T_len + 127) / 128;
     const int n_pb = (P + PBK - 1) / PBK;
     constexpr size_t lds_bytes = dq_ring_lds_bytes<DH, PBK>();

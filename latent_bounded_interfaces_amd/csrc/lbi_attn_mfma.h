@@ -393,7 +393,10 @@ int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T
     constexpr int rows_per_block = 256 / (DH / 8);
     hipLaunchKernelGGL((delta_kernel<T, DH>), dim3((unsigned)((T_len + rows_per_block - 1) / rows_per_block) * n_bh),
                        dim3(256), 0, stream, g, o32, delta, H, P, T_len);
-    if (DH == 64 && P > 4) launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    // directions per wave of the dQ kernel: as many as share one S tile, without idle slots for one or two directions
+    if (P == 1) launch_dq<T, DH, 1, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else if (P == 2) launch_dq<T, DH, 2, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else if (DH == 64 && P > 4) launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
     else launch_dq<T, DH, 4, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
     if (P >= 2) launch_dkdv_pair<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
     else launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
