@@ -313,6 +313,31 @@ def lbi_step_section(steps: int = 3) -> dict:
     return {"lbi_backward_step_bf16_L12_D768_B8_T1024_d64": measure_lbi_step(iters=steps)}
 
 
+def measure_scan(B: int, K: int, d: int, dtype, *, warmup=3, iters=10, device="cuda") -> dict:
+    """One fused suffix scan (all K suffix matrices + all K cotangents) of near-identity matrices, as the scan
+    benchmark feeds it; rates on the algorithmic flops and bytes."""
+    lib = _lib.load()
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    mats = torch.eye(d).expand(B, K, d, d) + torch.randn(B, K, d, d, generator=gen) * (0.01 / d) ** 0.5
+    mats = mats.to(dtype).to(device)
+    g = torch.randn(B, d, generator=gen).to(device)
+    out = torch.empty(B, K + 1, d, d, device=device)
+    cot = torch.empty(B, K + 1, d, device=device)
+
+    def call():
+        _lib.check(lib.lbi_suffix_scan_with_cotangents(mats.data_ptr(), g.data_ptr(), out.data_ptr(), cot.data_ptr(), B,
+                                                       K, d, _lib.dtype_code(mats.dtype), _lib.LBI_F32,
+                                                       _lib.current_stream_ptr(mats.device)),
+                   "lbi_suffix_scan_with_cotangents")
+
+    median_ms, best_ms, mean_ms, peak = time_call(call, warmup=warmup, iters=iters)
+    flops = B * (K - 1) * 2.0 * d ** 3
+    nbytes = B * K * d * d * (mats.element_size() + 4.0)
+    return {"B": B, "K": K, "d": d, "dtype": str(dtype).replace("torch.", ""), "median_ms": median_ms, "best_ms": best_ms,
+            "pullbacks_per_s": B * K / (median_ms * 1e-3), "tflops": flops / (median_ms * 1e-3) / 1e12,
+            "algorithmic_gbs": nbytes / (median_ms * 1e-3) / 1e9, "algorithmic_bytes": nbytes}
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
     ap.add_argument("--shapes", nargs="*", default=["1,8,128,64,4"], help="B,H,T,Dh,P tuples")
@@ -327,7 +352,14 @@ def main(argv=None) -> int:
     ap.add_argument("--basis", type=int, default=64, help="cotangent directions of the --region run")
     ap.add_argument("--lbi-step", action="store_true",
                     help="time the device work of one LBI scan backward step at the end-to-end configuration")
+    ap.add_argument("--scan", nargs="*", default=None, help="time the fused suffix scan instead: B,K,d tuples")
     args = ap.parse_args(argv)
+    if args.scan is not None:
+        for spec in args.scan:
+            B, K, d = (int(x) for x in spec.split(","))
+            print(json.dumps(measure_scan(B, K, d, getattr(torch, args.dtype), warmup=args.warmup, iters=args.iters)),
+                  flush=True)
+        return 0
     if args.lbi_step:
         print(json.dumps(measure_lbi_step(dtype=getattr(torch, args.dtype), warmup=args.warmup, iters=args.iters)),
               flush=True)

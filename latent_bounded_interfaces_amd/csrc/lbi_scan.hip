@@ -369,6 +369,85 @@ __global__ __launch_bounds__(512) void cotangent_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// Cotangent chain for d <= 128 (d a multiple of 4): the matrices are small, so a step is bound by the
+// latency of its loads unless they are issued a step ahead.  The matrix of step r - 1 is fetched into
+// registers while step r is multiplied out of an LDS copy, then stored to that copy (two barriers per
+// step, no load on the chain's critical path).  One workgroup of 256 threads per batch element; a row is
+// shared by the next power of two >= d / 4 lanes, 16 bytes each, folded with xor shuffles.
+// ---------------------------------------------------------------------------------------
+template <typename Tin>
+__global__ __launch_bounds__(256) void cotangent_staged_kernel(const Tin* __restrict__ mats, const float* __restrict__ g,
+                                                               float* __restrict__ out, int K, int d) {
+    extern __shared__ __align__(16) float lds[];  // [d * d] matrix copy, then [2][d] chain vectors
+    constexpr int NT = 256, MAXV = 16;            // 16-byte pieces of a matrix per thread: d * d / 4 / 256 <= 16
+    float* a_lds = lds;
+    float* vbuf = lds + d * d;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const Tin* mats_b = mats + (size_t)b * K * d * d;
+    float* out_b = out + (size_t)b * (K + 1) * d;
+    const int pieces = d * d / 4;
+    const int per_row = d / 4;
+    int lanes_per_row = 1;
+    while (lanes_per_row < per_row) lanes_per_row <<= 1;  // <= 32
+    const int rows_per_pass = NT / lanes_per_row;
+    const int sub = tid % lanes_per_row, row_in_pass = tid / lanes_per_row;
+
+    for (int i = tid; i < d; i += NT) {
+        const float val = g[(size_t)b * d + i];
+        vbuf[i] = val;
+        out_b[(size_t)K * d + i] = val;
+    }
+    f32x4 next[MAXV];
+    auto fetch = [&](int r) __attribute__((always_inline)) {
+        const Tin* a = mats_b + (size_t)r * d * d;
+#pragma unroll
+        for (int u = 0; u < MAXV; ++u) {
+            const int piece = tid + NT * u;
+            if (piece < pieces) next[u] = load4(a + 4 * piece);
+        }
+    };
+    auto commit = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < MAXV; ++u) {
+            const int piece = tid + NT * u;
+            if (piece < pieces) *reinterpret_cast<f32x4*>(a_lds + 4 * piece) = next[u];
+        }
+    };
+    if (K > 0) {
+        fetch(K - 1);
+        commit();
+    }
+    __syncthreads();
+    int cur = 0;
+    for (int r = K - 1; r >= 0; --r) {
+        if (r > 0) fetch(r - 1);
+        const float* v_old = vbuf + cur * d;
+        float* v_new = vbuf + (cur ^ 1) * d;
+        for (int row0 = 0; row0 < d; row0 += rows_per_pass) {
+            const int row = row0 + row_in_pass;
+            float acc = 0.0f;
+            if (row < d && sub < per_row) {
+                const f32x4 a4 = *reinterpret_cast<const f32x4*>(a_lds + row * d + 4 * sub);
+                const f32x4 v4 = *reinterpret_cast<const f32x4*>(v_old + 4 * sub);
+                acc = fmaf(a4[0], v4[0], acc);
+                acc = fmaf(a4[1], v4[1], acc);
+                acc = fmaf(a4[2], v4[2], acc);
+                acc = fmaf(a4[3], v4[3], acc);
+            }
+            for (int off = lanes_per_row >> 1; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+            if (row < d && sub == 0) {
+                v_new[row] = acc;
+                out_b[(size_t)r * d + row] = acc;
+            }
+        }
+        __syncthreads();  // every read of the matrix copy and of v_old is done, v_new is complete
+        if (r > 0) commit();
+        __syncthreads();
+        cur ^= 1;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Cotangent chain for d = 256, fp32: the HBM-bound case that matters.  One workgroup of
 // 8 waves per batch element; a wave takes rows wave, wave+8, ... (32 per step), one row
 // (1 KiB) per load instruction.  The matrices do not depend on the chain, so half a matrix
@@ -536,6 +615,17 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
     if (d == 256 && std::is_same<Tin, float>::value) {
         hipLaunchKernelGGL(cotangent256_kernel, dim3(B), dim3(512), 0, stream, static_cast<const float*>(mats),
                            static_cast<const float*>(g), static_cast<float*>(out), K);
+        LBI_HIP_CHECK(hipGetLastError());
+        return LBI_OK;
+    }
+    if (d % 4 == 0 && d <= 128) {
+        const size_t staged_bytes = ((size_t)d * d + 2 * d) * sizeof(float);  // <= 65 KB
+        auto kern = cotangent_staged_kernel<Tin>;
+        if (staged_bytes > 64 * 1024)
+            LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)staged_bytes));
+        hipLaunchKernelGGL(kern, dim3(B), dim3(256), staged_bytes, stream, static_cast<const Tin*>(mats),
+                           static_cast<const float*>(g), static_cast<float*>(out), K, d);
         LBI_HIP_CHECK(hipGetLastError());
         return LBI_OK;
     }
