@@ -556,6 +556,9 @@ int launch_mfma(const void* mats, void* out, const void* g, void* cot, int B, in
 template <typename Tin>
 int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, int d, hipStream_t stream);
 
+// batch size from which one workgroup per batch element already fills the chip (two per CU)
+constexpr int kWideBlockBatch = 512;
+
 // g / cot may be null (matrices only).  With them, the MFMA widths run the fused kernel;
 // other widths run the generic scan followed by the cotangent chain kernel.
 template <typename Tin>
@@ -586,8 +589,16 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
             }
             return launch_mfma<Tin, 256, 32, 64>(mats, out, g, cot, B, K, stream);
         }
-        case 128: return launch_mfma<Tin, 128, 32, 32>(mats, out, g, cot, B, K, stream);
-        case 64: return launch_mfma<Tin, 64, 32, 32>(mats, out, g, cot, B, K, stream);
+        // Column blocks of one batch element read the same matrices.  With few batch elements, narrow blocks give
+        // the chip enough workgroups, and the blocks of an element run side by side and share the matrices in L2.
+        // With many, they drift apart and fetch them again (measured 1.7x / 2.4x the input bytes at d = 64 / 128),
+        // so one workgroup then takes all columns.
+        case 128:
+            if (B >= kWideBlockBatch) return launch_mfma<Tin, 128, 32, 128>(mats, out, g, cot, B, K, stream);
+            return launch_mfma<Tin, 128, 32, 32>(mats, out, g, cot, B, K, stream);
+        case 64:
+            if (B >= kWideBlockBatch) return launch_mfma<Tin, 64, 32, 64>(mats, out, g, cot, B, K, stream);
+            return launch_mfma<Tin, 64, 32, 32>(mats, out, g, cot, B, K, stream);
         case 32: return launch_mfma<Tin, 32, 32, 32>(mats, out, g, cot, B, K, stream);
         default: break;
     }
