@@ -368,9 +368,11 @@ def region_input_pullback_basis(backend: Any, cache: Any, output_cotangent_basis
     if len(cache.layer_caches) != end - start:
         raise ValueError("cache.layer_caches does not match cache.layer_range")
     if end == start:
-        return output_cotangent_basis.clone()
-    g = _pull_back_region(backend, cache, output_cotangent_basis, kernel_mode, None)
-    return g.to(device=output_cotangent_basis.device, dtype=output_cotangent_basis.dtype)
+        return output_cotangent_basis.detach().clone()
+    # the result carries no autograd graph (weights and cache are constants here, as in the reference's extension)
+    with torch.no_grad():
+        g = _pull_back_region(backend, cache, output_cotangent_basis, kernel_mode, None)
+        return g.to(device=output_cotangent_basis.device, dtype=output_cotangent_basis.dtype)
 
 
 def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tensor, *,
@@ -404,6 +406,6 @@ def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tenso
 
 
 __all__ = [
-    "attn_heads_split", "attn_qkv_conv_pullback", "attn_qkv_pullback", "causal_conv1d_pullback", "gated_mlp_pullback", "rmsnorm_pullback",
-    "region_input_pullback_basis", "region_parameter_vjp", "rope_tables",
+    "attn_heads_split", "attn_qkv_conv_pullback", "attn_qkv_pullback", "causal_conv1d_pullback", "gated_mlp_pullback",
+    "rmsnorm_pullback", "region_input_pullback_basis", "region_parameter_vjp", "rope_tables",
 ]

@@ -214,6 +214,7 @@ def test_region_pullback_fp32_matches_autograd(case, device):
     assert got.shape == basis.shape and got.dtype == basis.dtype and got.is_cuda
     assert _max_rel(got.cpu(), want) <= 2e-5, _max_rel(got.cpu(), want)
     assert torch.equal(basis_d.cpu(), basis) and got.data_ptr() != basis_d.data_ptr()  # the caller's tensor is read only
+    assert not got.requires_grad and got.grad_fn is None  # no autograd graph although the weights require grad
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
