@@ -313,9 +313,9 @@ def lbi_step_section(steps: int = 3) -> dict:
     return {"lbi_backward_step_bf16_L12_D768_B8_T1024_d64": measure_lbi_step(iters=steps)}
 
 
-def measure_scan(B: int, K: int, d: int, dtype, *, warmup=3, iters=10, device="cuda") -> dict:
-    """One fused suffix scan (all K suffix matrices + all K cotangents) of near-identity matrices, as the scan
-    benchmark feeds it; rates on the algorithmic flops and bytes."""
+def measure_scan(B: int, K: int, d: int, dtype, *, warmup=3, iters=10, device="cuda", matrices_only=False) -> dict:
+    """One suffix scan of near-identity matrices, as the scan benchmark feeds it: all K suffix matrices and all K
+    cotangents in one call, or (``matrices_only``) the matrices alone; rates on the algorithmic flops and bytes."""
     lib = _lib.load()
     gen = torch.Generator(device="cpu").manual_seed(0)
     mats = torch.eye(d).expand(B, K, d, d) + torch.randn(B, K, d, d, generator=gen) * (0.01 / d) ** 0.5
@@ -325,6 +325,10 @@ def measure_scan(B: int, K: int, d: int, dtype, *, warmup=3, iters=10, device="c
     cot = torch.empty(B, K + 1, d, device=device)
 
     def call():
+        if matrices_only:
+            _lib.check(lib.lbi_suffix_scan(mats.data_ptr(), out.data_ptr(), B, K, d, _lib.dtype_code(mats.dtype),
+                                           _lib.LBI_F32, _lib.current_stream_ptr(mats.device)), "lbi_suffix_scan")
+            return
         _lib.check(lib.lbi_suffix_scan_with_cotangents(mats.data_ptr(), g.data_ptr(), out.data_ptr(), cot.data_ptr(), B,
                                                        K, d, _lib.dtype_code(mats.dtype), _lib.LBI_F32,
                                                        _lib.current_stream_ptr(mats.device)),
@@ -333,7 +337,8 @@ def measure_scan(B: int, K: int, d: int, dtype, *, warmup=3, iters=10, device="c
     median_ms, best_ms, mean_ms, peak = time_call(call, warmup=warmup, iters=iters)
     flops = B * (K - 1) * 2.0 * d ** 3
     nbytes = B * K * d * d * (mats.element_size() + 4.0)
-    return {"B": B, "K": K, "d": d, "dtype": str(dtype).replace("torch.", ""), "median_ms": median_ms, "best_ms": best_ms,
+    return {"B": B, "K": K, "d": d, "dtype": str(dtype).replace("torch.", ""), "matrices_only": matrices_only,
+            "median_ms": median_ms, "best_ms": best_ms,
             "pullbacks_per_s": B * K / (median_ms * 1e-3), "tflops": flops / (median_ms * 1e-3) / 1e12,
             "algorithmic_gbs": nbytes / (median_ms * 1e-3) / 1e9, "algorithmic_bytes": nbytes}
 
@@ -353,12 +358,13 @@ def main(argv=None) -> int:
     ap.add_argument("--lbi-step", action="store_true",
                     help="time the device work of one LBI scan backward step at the end-to-end configuration")
     ap.add_argument("--scan", nargs="*", default=None, help="time the fused suffix scan instead: B,K,d tuples")
+    ap.add_argument("--matrices-only", action="store_true", help="--scan: the suffix matrices without the cotangents")
     args = ap.parse_args(argv)
     if args.scan is not None:
         for spec in args.scan:
             B, K, d = (int(x) for x in spec.split(","))
-            print(json.dumps(measure_scan(B, K, d, getattr(torch, args.dtype), warmup=args.warmup, iters=args.iters)),
-                  flush=True)
+            print(json.dumps(measure_scan(B, K, d, getattr(torch, args.dtype), warmup=args.warmup, iters=args.iters,
+                                          matrices_only=args.matrices_only)), flush=True)
         return 0
     if args.lbi_step:
         print(json.dumps(measure_lbi_step(dtype=getattr(torch, args.dtype), warmup=args.warmup, iters=args.iters)),
