@@ -369,48 +369,55 @@ __global__ __launch_bounds__(512) void cotangent_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// Cotangent chain for d <= 128 (d a multiple of 4): the matrices are small, so a step is bound by the
-// latency of its loads unless they are issued a step ahead.  The matrix of step r - 1 is fetched into
-// registers while step r is multiplied out of an LDS copy, then stored to that copy (two barriers per
-// step, no load on the chain's critical path).  One workgroup of 256 threads per batch element; a row is
-// shared by the next power of two >= d / 4 lanes, 16 bytes each, folded with xor shuffles.
+// Cotangent chain for matrices that fit in LDS in their storage type (rows a multiple of 16 bytes; fp32 up to
+// d = 180, 16-bit up to d = 256): a step is bound by the latency of its loads unless they are issued a step ahead.
+// The matrix of step r - 1 is fetched into registers while step r is multiplied out of an LDS copy, then
+// stored to that copy (two barriers per step, no load on the chain's critical path).  One workgroup of 256
+// threads per batch element; a thread multiplies a run of 16-byte pieces of one row, the (at most 32) lanes of a
+// row are folded with xor shuffles.
 // ---------------------------------------------------------------------------------------
 template <typename Tin>
 __global__ __launch_bounds__(256) void cotangent_staged_kernel(const Tin* __restrict__ mats, const float* __restrict__ g,
                                                                float* __restrict__ out, int K, int d) {
-    extern __shared__ __align__(16) float lds[];  // [d * d] matrix copy, then [2][d] chain vectors
-    constexpr int NT = 256, MAXV = 16;            // 16-byte pieces of a matrix per thread: d * d / 4 / 256 <= 16
-    float* a_lds = lds;
-    float* vbuf = lds + d * d;
+    constexpr int NT = 256, MAXV = 32;            // 16-byte pieces of a matrix per thread (128 KB / 16 / 256)
+    constexpr int EPP = 16 / (int)sizeof(Tin);    // elements per piece: 4 (fp32) or 8 (16-bit)
+    typedef unsigned int raw4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) char lds_raw[];  // matrix copy [d * d] in Tin, then [2][d] fp32 chain vectors
+    Tin* a_lds = reinterpret_cast<Tin*>(lds_raw);
+    float* vbuf = reinterpret_cast<float*>(lds_raw + (size_t)d * d * sizeof(Tin));
     const int b = blockIdx.x, tid = threadIdx.x;
     const Tin* mats_b = mats + (size_t)b * K * d * d;
     float* out_b = out + (size_t)b * (K + 1) * d;
-    const int pieces = d * d / 4;
-    const int per_row = d / 4;
-    int lanes_per_row = 1;
-    while (lanes_per_row < per_row) lanes_per_row <<= 1;  // <= 32
-    const int rows_per_pass = NT / lanes_per_row;
-    const int sub = tid % lanes_per_row, row_in_pass = tid / lanes_per_row;
+    const int pieces = d * d / EPP;
+    const int per_row = d / EPP;
+    // A row is shared by `parts` adjacent lanes (a power of two, as many as 256 threads allow), each taking a run
+    // of `ppp` pieces; lanes start their runs at different pieces so that a wave's 16-byte reads spread over banks.
+    int parts = 1;
+    while (2 * parts * d <= NT && 2 * parts <= per_row) parts <<= 1;
+    const int ppp = (per_row + parts - 1) / parts;
+    const int row = tid / parts, part = tid % parts;
 
     for (int i = tid; i < d; i += NT) {
         const float val = g[(size_t)b * d + i];
         vbuf[i] = val;
         out_b[(size_t)K * d + i] = val;
     }
-    f32x4 next[MAXV];
+    raw4 next[MAXV];
     auto fetch = [&](int r) __attribute__((always_inline)) {
-        const Tin* a = mats_b + (size_t)r * d * d;
+        const raw4* a = reinterpret_cast<const raw4*>(mats_b + (size_t)r * d * d);
 #pragma unroll
         for (int u = 0; u < MAXV; ++u) {
             const int piece = tid + NT * u;
-            if (piece < pieces) next[u] = load4(a + 4 * piece);
+            if (NT * u >= pieces) break;  // uniform: small matrices leave after one or two rounds
+            if (piece < pieces) next[u] = a[piece];
         }
     };
     auto commit = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < MAXV; ++u) {
             const int piece = tid + NT * u;
-            if (piece < pieces) *reinterpret_cast<f32x4*>(a_lds + 4 * piece) = next[u];
+            if (NT * u >= pieces) break;
+            if (piece < pieces) reinterpret_cast<raw4*>(a_lds)[piece] = next[u];
         }
     };
     if (K > 0) {
@@ -423,22 +430,31 @@ __global__ __launch_bounds__(256) void cotangent_staged_kernel(const Tin* __rest
         if (r > 0) fetch(r - 1);
         const float* v_old = vbuf + cur * d;
         float* v_new = vbuf + (cur ^ 1) * d;
-        for (int row0 = 0; row0 < d; row0 += rows_per_pass) {
-            const int row = row0 + row_in_pass;
-            float acc = 0.0f;
-            if (row < d && sub < per_row) {
-                const f32x4 a4 = *reinterpret_cast<const f32x4*>(a_lds + row * d + 4 * sub);
-                const f32x4 v4 = *reinterpret_cast<const f32x4*>(v_old + 4 * sub);
-                acc = fmaf(a4[0], v4[0], acc);
-                acc = fmaf(a4[1], v4[1], acc);
-                acc = fmaf(a4[2], v4[2], acc);
-                acc = fmaf(a4[3], v4[3], acc);
+        float acc = 0.0f;
+        if (row < d) {
+            const Tin* a_row = a_lds + row * d;
+#pragma unroll 4
+            for (int i = 0; i < ppp; ++i) {
+                int rot = i + row;
+                rot -= (rot / ppp) * ppp;
+                const int piece = part * ppp + rot;
+                if (piece < per_row) {
+#pragma unroll
+                    for (int q = 0; q < EPP / 4; ++q) {
+                        const f32x4 a4 = load4(a_row + EPP * piece + 4 * q);
+                        const f32x4 v4 = *reinterpret_cast<const f32x4*>(v_old + EPP * piece + 4 * q);
+                        acc = fmaf(a4[0], v4[0], acc);
+                        acc = fmaf(a4[1], v4[1], acc);
+                        acc = fmaf(a4[2], v4[2], acc);
+                        acc = fmaf(a4[3], v4[3], acc);
+                    }
+                }
             }
-            for (int off = lanes_per_row >> 1; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
-            if (row < d && sub == 0) {
-                v_new[row] = acc;
-                out_b[(size_t)r * d + row] = acc;
-            }
+        }
+        for (int off = parts >> 1; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (row < d && part == 0) {
+            v_new[row] = acc;
+            out_b[(size_t)r * d + row] = acc;
         }
         __syncthreads();  // every read of the matrix copy and of v_old is done, v_new is complete
         if (r > 0) commit();
@@ -629,8 +645,10 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
         LBI_HIP_CHECK(hipGetLastError());
         return LBI_OK;
     }
-    if (d % 4 == 0 && d <= 128) {
-        const size_t staged_bytes = ((size_t)d * d + 2 * d) * sizeof(float);  // <= 65 KB
+    const size_t matrix_bytes = (size_t)d * d * sizeof(Tin);
+    constexpr int per_piece = 16 / (int)sizeof(Tin);  // elements in 16 bytes
+    if (d % per_piece == 0 && matrix_bytes <= 128 * 1024 && d / per_piece <= 64) {
+        const size_t staged_bytes = matrix_bytes + (size_t)2 * d * sizeof(float);  // <= 130 KB
         auto kern = cotangent_staged_kernel<Tin>;
         if (staged_bytes > 64 * 1024)
             LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
