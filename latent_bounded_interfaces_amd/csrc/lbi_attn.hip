@@ -5,6 +5,9 @@
 #include "lbi_attn_dkdv128.h"
 #include "lbi_attn_dkdv_pair.h"
 #include "lbi_attn_dq128.h"
+#include "lbi_attn_small.h"
+
+#include <cstdlib>
 
 namespace lbi {
 namespace {
@@ -51,6 +54,20 @@ extern "C" int lbi_attn_pullback(const void* q, const void* k, const void* v, co
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     float* ws = static_cast<float*>(workspace);
     const int b = (int)B, h = (int)H, t = (int)T, dh = (int)Dh, p = (int)P;
+    // Short sequences: one launch that does everything per (b, h, direction).  LBI_ATTN_SMALL=0 keeps the
+    // four-kernel path.
+    static const bool small_path = !(std::getenv("LBI_ATTN_SMALL") && std::atoi(std::getenv("LBI_ATTN_SMALL")) == 0);
+    if (small_path && attn_small::supports(t, dh, dtype)) {
+        const size_t align = dtype_size(dtype) * 8;
+        if (reinterpret_cast<uintptr_t>(q) % align || reinterpret_cast<uintptr_t>(k) % align ||
+            reinterpret_cast<uintptr_t>(v) % align || reinterpret_cast<uintptr_t>(d_out) % align ||
+            reinterpret_cast<uintptr_t>(dq) % 8 || reinterpret_cast<uintptr_t>(dk) % 8 ||
+            reinterpret_cast<uintptr_t>(dv) % 8)
+            return fail(LBI_ERR_INVALID, "lbi_attn_pullback: tensors must be 16-byte aligned");
+        return dtype == LBI_F16
+                   ? attn_small::launch<_Float16>(q, k, v, d_out, dq, dk, dv, b, h, t, p, softmax_scale, causal, stream)
+                   : attn_small::launch<bf16_raw>(q, k, v, d_out, dq, dk, dv, b, h, t, p, softmax_scale, causal, stream);
+    }
     if (attn_mfma::supports(t, dh, dtype)) {
         const size_t align = dtype_size(dtype) * 8;  // 16-byte vector loads on every row
         if (reinterpret_cast<uintptr_t>(q) % align || reinterpret_cast<uintptr_t>(k) % align ||

@@ -68,7 +68,8 @@ def test_fp32_matches_oracle(seed, shape, basis, causal, device):
         assert torch.allclose(a.double(), c, atol=2e-5, rtol=2e-5)
 
 
-# 16-bit storage: the MFMA kernels (T % 64 == 0, Dh in {64, 128}) and the generic ones otherwise.
+# 16-bit storage: the MFMA kernels (T % 64 == 0, Dh in {64, 128}; one fused launch for Dh = 64, T <= 128) and the
+# generic ones otherwise.
 # (121, (1, 2, 16, 64), P) are the reference's fp16 cases (tests/test_cuda_attention_pullback.py:178-243);
 # (8, 8, 128, 64) with P=4 is the reference benchmark shape.
 LOWP_CASES = [
@@ -80,6 +81,9 @@ LOWP_CASES = [
     # head dims below 128 that are not 64: zero-padded onto the matrix-core kernels (with the length, if causal)
     (24, (1, 2, 128, 32), 3), (25, (2, 1, 192, 96), 2), (26, (1, 2, 70, 80), 2), (27, (1, 1, 64, 8), 1),
     (28, (1, 1, 128, 160), 2),  # past 128: generic kernels
+    # head dim 64, length a multiple of 32 up to 128: the single-launch kernel (so are 11, 16, 17 above and, once
+    # padded, the causal runs of 21, 23, 24, 27)
+    (29, (1, 2, 32, 64), 3), (30, (3, 1, 128, 64), 1), (31, (2, 3, 96, 64), 5),
 ]
 
 
@@ -96,6 +100,30 @@ def test_low_precision_matches_oracle(seed, shape, basis, causal, dtype, device)
         assert a.shape == g.shape and a.dtype == dtype
         assert _max_rel(a, c) <= 2e-2, (name, _max_rel(a, c))  # bar: <= 2e-2 against the fp32 path
         assert torch.allclose(a.float(), c, atol=3e-2 * float(c.abs().max()), rtol=3e-2), name
+
+
+def test_four_kernel_path_at_short_lengths_in_subprocess(device):
+    """LBI_ATTN_SMALL=0 sends short sequences through the four-kernel path; it meets the same bar."""
+    import os
+    import subprocess
+    import sys
+
+    code = (
+        "import math, sys, torch; sys.path.insert(0, %r);"
+        "from oracle import attention as o;"
+        "from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis as f;"
+        "worst = 0.0\n"
+        "for shape, basis, causal in (((2, 2, 64, 64), 2, True), ((8, 8, 128, 64), 4, True), ((1, 2, 128, 64), 3, False)):\n"
+        "    q, k, v, g = o.make_attention_inputs(*shape, basis, dtype=torch.float16, seed=41)\n"
+        "    got = f(q.cuda(), k.cuda(), v.cuda(), g.cuda(), softmax_scale=0.125, causal=causal, kernel_mode='hip')\n"
+        "    truth = o.attention_pullback_blocked(q, k, v, g, softmax_scale=0.125, causal=causal, dtype=torch.float32)\n"
+        "    for a, c in zip(got, truth):\n"
+        "        worst = max(worst, float((a.cpu().double() - c.double()).abs().max() / c.double().abs().max()))\n"
+        "print(worst); sys.exit(0 if 0.0 < worst <= 2e-2 else 1)"
+    ) % str(Path(__file__).resolve().parents[1])
+    env = dict(os.environ, LBI_ATTN_SMALL="0")
+    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stdout + res.stderr
 
 
 def test_modes_and_contract(device):
