@@ -466,9 +466,9 @@ __global__ __launch_bounds__(256) void cotangent_staged_kernel(const Tin* __rest
 // ---------------------------------------------------------------------------------------
 // Cotangent chain for d = 256, fp32: the HBM-bound case that matters.  One workgroup of
 // 8 waves per batch element; a wave takes rows wave, wave+8, ... (32 per step), one row
-// (1 KiB) per load instruction.  The matrices do not depend on the chain, so half a matrix
-// per wave is always in flight in registers (two 16-row buffers, 128 KiB per workgroup)
-// while the other half is multiplied.  The 32 partial sums of a lane are folded across
+// (1 KiB) per load instruction.  The matrices do not depend on the chain, so a wave keeps its
+// 32 rows of the next matrix in flight in registers (248 KiB per workgroup) while the current
+// ones are multiplied.  The 32 partial sums of a lane are folded across
 // the 64 lanes with a halving butterfly (31 exchanges instead of 32 x 6).
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(512) void cotangent256_kernel(const float* __restrict__ mats,
@@ -487,31 +487,30 @@ __global__ __launch_bounds__(512) void cotangent256_kernel(const float* __restri
         out_b[(size_t)K * D + tid] = val;
     }
     if (K == 0) return;
-    // 16 rows: wave + 8 * (16 * half + i), columns 4 * lane .. 4 * lane + 3
-    auto load_half = [&](f32x4 (&dst)[16], int r, int half) {
-        const float* base = mats_b + (size_t)r * D * D + (size_t)(wave + 128 * half) * D;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = *reinterpret_cast<const f32x4*>(base + (size_t)(8 * i) * D + 4 * lane);
+    // Row wave + 8 * i of matrix r, columns 4 * lane .. 4 * lane + 3.
+    auto load_row = [&](int r, int i) {
+        return *reinterpret_cast<const f32x4*>(mats_b + (size_t)r * D * D + (size_t)(wave + 8 * i) * D + 4 * lane);
     };
     // LDS writes visible to the workgroup; loads already in flight are NOT waited for
     // (a full __syncthreads would drain them together with the stores of the step).
     auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-    f32x4 buf_a[16], buf_b[16];
-    load_half(buf_a, K - 1, 0);
+    f32x4 buf[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) buf[i] = load_row(K - 1, i);
     lds_barrier();
     int cur = 0;
     for (int r = K - 1; r >= 0; --r) {
         const f32x4 vv = *reinterpret_cast<const f32x4*>(&vbuf[cur][4 * lane]);
+        const int r_next = r > 0 ? r - 1 : 0;  // a harmless re-read at the end
         float vals[32];
-        load_half(buf_b, r, 1);
+        // Each register is refilled with the same row of the next matrix as soon as it has been used: 31 of the
+        // wave's 32 rows are in flight at any time.
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
-            vals[i] = fmaf(buf_a[i][3], vv[3], fmaf(buf_a[i][2], vv[2], fmaf(buf_a[i][1], vv[1], buf_a[i][0] * vv[0])));
-        load_half(buf_a, r > 0 ? r - 1 : 0, 0);  // next step's first half (a harmless re-read at the end)
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-            vals[16 + i] =
-                fmaf(buf_b[i][3], vv[3], fmaf(buf_b[i][2], vv[2], fmaf(buf_b[i][1], vv[1], buf_b[i][0] * vv[0])));
+        for (int i = 0; i < 32; ++i) {
+            vals[i] = fmaf(buf[i][3], vv[3], fmaf(buf[i][2], vv[2], fmaf(buf[i][1], vv[1], buf[i][0] * vv[0])));
+            buf[i] = load_row(r_next, i);
+            __builtin_amdgcn_sched_barrier(0);  // keep the refill next to the use
+        }
         // Halving butterfly: after the stage with mask M a lane keeps the half of its values
         // selected by its bit M; at the end lane l holds row index l >> 1 summed over all lanes.
         auto stage = [&](auto half_tag) {
