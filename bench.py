@@ -15,7 +15,9 @@ Prints ONE JSON line.  Besides the contract keys it carries
                       host cores of the same box on a bounded batch slice;
 * ``extra``         - the other measured variants (bf16 storage, cotangent-only chain,
                       attention input-pullback, region-level input pullback) with their own
-                      roofline figures.
+                      roofline figures; the two attention entries carry a ``cpu_baseline`` of
+                      their own (the reference's per-direction SDPA + autograd loop, fp32, on a
+                      bounded sample).
 """
 from __future__ import annotations
 
@@ -103,6 +105,46 @@ def _cpu_baseline(sample_batch: int) -> dict:
         "sample": f"B={sample_batch} of {SCAN_B} batch elements, K={SCAN_K}, d={SCAN_D}, fp32, "
                   f"log-depth torch scan + mat-vecs, {dt:.2f} s wall",
     }
+
+
+def _cpu_attention_baselines() -> dict:
+    """The reference's CPU path for the attention pullback (one SDPA forward + autograd backward per direction,
+    fp32) on bounded samples of the two attention workloads; rates in algorithmic TFLOP/s."""
+    import math
+    import statistics as st
+
+    import torch
+
+    from oracle import attention as oattn
+
+    def flops(b, h, t, dh, p):
+        return b * h * (t * (t + 1) / 2) * 2 * dh * (1 + 4 * p)
+
+    cores = int(torch.get_num_threads())
+    out = {}
+    # long-context workload: 4 of its 64 (batch, head) pairs, all 16 directions
+    q, k, v, g = oattn.make_attention_inputs(1, 4, 4096, 128, 16, dtype=torch.float32, seed=0)
+    t0 = time.perf_counter()
+    oattn.attention_pullback_sdpa_loop(q, k, v, g, softmax_scale=128 ** -0.5, causal=True)
+    dt = time.perf_counter() - t0
+    out["attn_pullback_bf16_B4_H16_T4096_Dh128_P16"] = {
+        "value": flops(1, 4, 4096, 128, 16) / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"4 of the 64 (batch, head) pairs, all 16 directions, fp32, per-direction SDPA + autograd, "
+                  f"{dt:.2f} s wall",
+    }
+    # the small workload runs whole
+    q, k, v, g = oattn.make_attention_inputs(8, 8, 128, 64, 4, dtype=torch.float32, seed=0)
+    times = []
+    for _ in range(7):
+        t0 = time.perf_counter()
+        oattn.attention_pullback_sdpa_loop(q, k, v, g, softmax_scale=1.0 / math.sqrt(64), causal=True)
+        times.append(time.perf_counter() - t0)
+    dt = st.median(times[2:])
+    out["attn_pullback_fp16_B8_H8_T128_Dh64_P4"] = {
+        "value": flops(8, 8, 128, 64, 4) / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"the whole workload in fp32, per-direction SDPA + autograd, median of 5 runs, {dt * 1e3:.1f} ms",
+    }
+    return out
 
 
 def main() -> int:
@@ -258,6 +300,10 @@ def main() -> int:
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _cpu_baseline(args.cpu_sample_batch)
+        if "extra" in result:
+            for key, base in _cpu_attention_baselines().items():
+                if key in result["extra"]:
+                    result["extra"][key]["cpu_baseline"] = base
 
     print(json.dumps(result))
     return 0
