@@ -24,6 +24,13 @@ int check_attn_dims(int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P, int 
     return LBI_OK;
 }
 
+// Short sequences: one launch that does everything per (b, h, direction), no workspace.  LBI_ATTN_SMALL=0 keeps
+// the four-kernel path.
+bool use_small_path(int T_len, int dh, int dtype) {
+    static const bool enabled = !(std::getenv("LBI_ATTN_SMALL") && std::atoi(std::getenv("LBI_ATTN_SMALL")) == 0);
+    return enabled && attn_small::supports(T_len, dh, dtype);
+}
+
 }  // namespace
 }  // namespace lbi
 
@@ -32,6 +39,7 @@ extern "C" size_t lbi_attn_pullback_workspace_bytes(int64_t B, int64_t H, int64_
     using namespace lbi;
     if (check_attn_dims(B, H, T, Dh, P, dtype) != LBI_OK) return 0;
     if (B == 0 || H == 0 || T == 0 || Dh == 0 || P == 0) return 0;
+    if (use_small_path((int)T, (int)Dh, dtype)) return 0;
     const size_t floats = attn_mfma::supports((int)T, (int)Dh, dtype) ? attn_mfma::workspace_floats(B, H, T, Dh, P)
                                                                      : attn_generic::workspace_floats(B, H, T, P);
     return (floats * sizeof(float) + 255) & ~(size_t)255;
@@ -46,18 +54,15 @@ extern "C" int lbi_attn_pullback(const void* q, const void* k, const void* v, co
     if (B == 0 || H == 0 || T == 0 || Dh == 0 || P == 0) return LBI_OK;
     if (!q || !k || !v || !d_out || !dq || !dk || !dv) return fail(LBI_ERR_INVALID, "lbi_attn_pullback: null tensor pointer");
     const size_t need = lbi_attn_pullback_workspace_bytes(B, H, T, Dh, P, dtype);
-    if (!workspace || workspace_bytes < need)
+    if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(LBI_ERR_WORKSPACE, "lbi_attn_pullback: workspace of %zu bytes needed, %zu given", need,
                     workspace_bytes);
-    if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+    if (need > 0 && reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
         return fail(LBI_ERR_WORKSPACE, "lbi_attn_pullback: workspace must be 16-byte aligned");
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     float* ws = static_cast<float*>(workspace);
     const int b = (int)B, h = (int)H, t = (int)T, dh = (int)Dh, p = (int)P;
-    // Short sequences: one launch that does everything per (b, h, direction).  LBI_ATTN_SMALL=0 keeps the
-    // four-kernel path.
-    static const bool small_path = !(std::getenv("LBI_ATTN_SMALL") && std::atoi(std::getenv("LBI_ATTN_SMALL")) == 0);
-    if (small_path && attn_small::supports(t, dh, dtype)) {
+    if (use_small_path(t, dh, dtype)) {
         const size_t align = dtype_size(dtype) * 8;
         if (reinterpret_cast<uintptr_t>(q) % align || reinterpret_cast<uintptr_t>(k) % align ||
             reinterpret_cast<uintptr_t>(v) % align || reinterpret_cast<uintptr_t>(d_out) % align ||

@@ -82,16 +82,18 @@ def attention_input_pullback_basis(
     d_out = output_cotangent_basis.contiguous()
     bsz, heads, seqlen, head_dim = q.shape
     if q.dtype in (torch.float16, torch.bfloat16) and d_out.numel() and seqlen > _MFMA_SEQ_MULTIPLE // 2:
-        # The matrix-core kernels take head dims 64 and 128 and sequence lengths that are multiples of 64; everything
-        # else runs on the generic kernels, at a small fraction of their speed.  Two paddings are exact:
+        # The matrix-core kernels take head dims 64 and 128 and sequence lengths that are multiples of 64 (of 32 at
+        # head dim 64 up to 128 positions); everything else runs on the generic kernels, at a small fraction of their speed.  Two paddings are exact:
         # * zero columns appended to the head dim add nothing to any dot product (the scale is passed explicitly)
         #   and receive zero cotangents;
         # * under the causal mask, zero rows appended after the sequence are invisible to every real query, and as
         #   queries they carry a zero cotangent, so they add nothing to dK or dV.
         wide_dim = next((w for w in _MFMA_HEAD_DIMS if w >= head_dim), head_dim)
-        ragged = seqlen % _MFMA_SEQ_MULTIPLE != 0
-        long_seq = seqlen + (_MFMA_SEQ_MULTIPLE - seqlen % _MFMA_SEQ_MULTIPLE) if (ragged and causal) else seqlen
-        if (wide_dim != head_dim or long_seq != seqlen) and long_seq % _MFMA_SEQ_MULTIPLE == 0 \
+        # head dim 64 up to 128 positions: the single-launch kernel takes multiples of 32
+        multiple = 32 if (wide_dim == 64 and seqlen <= 128) else _MFMA_SEQ_MULTIPLE
+        ragged = seqlen % multiple != 0
+        long_seq = seqlen + (multiple - seqlen % multiple) if (ragged and causal) else seqlen
+        if (wide_dim != head_dim or long_seq != seqlen) and long_seq % multiple == 0 \
                 and wide_dim in _MFMA_HEAD_DIMS:
             pads = (0, wide_dim - head_dim, 0, long_seq - seqlen)
             padded = [torch.nn.functional.pad(t, pads) for t in (q, k, v, d_out)]
@@ -106,11 +108,12 @@ def attention_input_pullback_basis(
     lib = _lib.load()
     with torch.cuda.device(q.device):
         need = int(lib.lbi_attn_pullback_workspace_bytes(bsz, heads, seqlen, head_dim, basis, dtype))
-        workspace = torch.empty(max(need, 256), device=q.device, dtype=torch.uint8)
+        # short sequences run as one launch that needs none
+        workspace = torch.empty(need, device=q.device, dtype=torch.uint8) if need > 0 else None
         status = lib.lbi_attn_pullback(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(),
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-            workspace.data_ptr(), workspace.numel(),
+            workspace.data_ptr() if need > 0 else None, need,
             bsz, heads, seqlen, head_dim, basis,
             float(softmax_scale), int(bool(causal)), dtype, _lib.current_stream_ptr(q.device),
         )

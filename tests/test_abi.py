@@ -75,6 +75,13 @@ def test_region_and_norm_entry_points_validate_on_the_host():
     assert lib.lbi_matrix_norms(one, one, one, None, 0, 4, 256, f32, None) == -4
     assert b"workspace" in lib.lbi_last_error()
     assert lib.lbi_matrix_norms(None, None, None, None, 0, 0, 16, f32, None) == 0
+    # attention: short 16-bit sequences at head dim 64 run as one launch and need no workspace
+    f16 = _lib.LBI_F16
+    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f16) == 0
+    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 256, 64, 4, f16) == 4 * (64 * 256 + 256 * 256 + 64 * 256 * 64)
+    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f32) > 0
+    assert lib.lbi_attn_pullback(one, one, one, one, one, one, one, None, 0, 8, 8, 256, 64, 4, 0.125, 1, f16, None) == -4
+    assert b"workspace" in lib.lbi_last_error()
 
 
 def test_wrappers_reject_bad_input_before_touching_the_device():
