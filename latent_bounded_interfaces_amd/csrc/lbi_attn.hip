@@ -70,8 +70,8 @@ extern "C" int lbi_attn_pullback(const void* q, const void* k, const void* v, co
             reinterpret_cast<uintptr_t>(dv) % 8)
             return fail(LBI_ERR_INVALID, "lbi_attn_pullback: tensors must be 16-byte aligned");
         return dtype == LBI_F16
-                   ? attn_small::launch<_Float16>(q, k, v, d_out, dq, dk, dv, b, h, t, p, softmax_scale, causal, stream)
-                   : attn_small::launch<bf16_raw>(q, k, v, d_out, dq, dk, dv, b, h, t, p, softmax_scale, causal, stream);
+                   ? attn_small::launch<_Float16>(q, k, v, d_out, dq, dk, dv, b, h, t, dh, p, softmax_scale, causal, stream)
+                   : attn_small::launch<bf16_raw>(q, k, v, d_out, dq, dk, dv, b, h, t, dh, p, softmax_scale, causal, stream);
     }
     if (attn_mfma::supports(t, dh, dtype)) {
         const size_t align = dtype_size(dtype) * 8;  // 16-byte vector loads on every row

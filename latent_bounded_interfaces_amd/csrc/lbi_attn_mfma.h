@@ -1,6 +1,6 @@
 // Attention input-pullback, MFMA path: fp16 / bf16 storage, head dim 64 or 128,
-// T a multiple of 64, causal or not, fp32 accumulation.  (Head dim 64 with T <= 128 runs as one
-// launch instead: lbi_attn_small.h, built from the same fragments.)
+// T a multiple of 64, causal or not, fp32 accumulation.  (Short sequences run as one launch
+// instead: lbi_attn_small.h, built from the same fragments.)
 //
 // Four kernels per call, all atomic-free (every output tile has one owner, sums run
 // in a fixed order, so reruns are bit-identical):

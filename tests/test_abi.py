@@ -78,9 +78,11 @@ def test_region_and_norm_entry_points_validate_on_the_host():
     # attention: short 16-bit sequences at head dim 64 run as one launch and need no workspace
     f16 = _lib.LBI_F16
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f16) == 0
-    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 256, 64, 4, f16) == 4 * (64 * 256 + 256 * 256 + 64 * 256 * 64)
+    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 256, 64, 4, f16) == 0
+    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 128, 4, f16) == 0
+    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 320, 64, 4, f16) == 4 * (64 * 320 + 256 * 320 + 64 * 320 * 64)
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f32) > 0
-    assert lib.lbi_attn_pullback(one, one, one, one, one, one, one, None, 0, 8, 8, 256, 64, 4, 0.125, 1, f16, None) == -4
+    assert lib.lbi_attn_pullback(one, one, one, one, one, one, one, None, 0, 8, 8, 320, 64, 4, 0.125, 1, f16, None) == -4
     assert b"workspace" in lib.lbi_last_error()
 
 

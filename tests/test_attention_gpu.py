@@ -81,9 +81,10 @@ LOWP_CASES = [
     # head dims below 128 that are not 64: zero-padded onto the matrix-core kernels (with the length, if causal)
     (24, (1, 2, 128, 32), 3), (25, (2, 1, 192, 96), 2), (26, (1, 2, 70, 80), 2), (27, (1, 1, 64, 8), 1),
     (28, (1, 1, 128, 160), 2),  # past 128: generic kernels
-    # head dim 64, length a multiple of 32 up to 128: the single-launch kernel (so are 11, 16, 17 above and, once
-    # padded, the causal runs of 21, 23, 24, 27)
-    (29, (1, 2, 32, 64), 3), (30, (3, 1, 128, 64), 1), (31, (2, 3, 96, 64), 5),
+    # lengths that are multiples of 32, up to 256 at head dim 64 and 128 at head dim 128: the single-launch kernel
+    # (so are 11, 12, 13, 16, 17, 19 above and, once padded, the causal runs of 21, 23, 24, 27)
+    (29, (1, 2, 32, 64), 3), (30, (3, 1, 128, 64), 1), (31, (2, 3, 96, 64), 5), (32, (1, 2, 160, 64), 2),
+    (33, (2, 1, 64, 128), 3), (34, (1, 1, 96, 128), 2), (35, (1, 2, 224, 64), 1), (36, (2, 2, 256, 64), 4),
 ]
 
 
@@ -113,10 +114,11 @@ def test_four_kernel_path_at_short_lengths_in_subprocess(device):
         "from oracle import attention as o;"
         "from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis as f;"
         "worst = 0.0\n"
-        "for shape, basis, causal in (((2, 2, 64, 64), 2, True), ((8, 8, 128, 64), 4, True), ((1, 2, 128, 64), 3, False)):\n"
+        "for shape, basis, causal in (((2, 2, 64, 64), 2, True), ((8, 8, 128, 64), 4, True), ((1, 2, 128, 64), 3, False),"
+        " ((1, 2, 256, 64), 2, True), ((1, 2, 128, 128), 2, True)):\n"
         "    q, k, v, g = o.make_attention_inputs(*shape, basis, dtype=torch.float16, seed=41)\n"
-        "    got = f(q.cuda(), k.cuda(), v.cuda(), g.cuda(), softmax_scale=0.125, causal=causal, kernel_mode='hip')\n"
-        "    truth = o.attention_pullback_blocked(q, k, v, g, softmax_scale=0.125, causal=causal, dtype=torch.float32)\n"
+        "    got = f(q.cuda(), k.cuda(), v.cuda(), g.cuda(), softmax_scale=shape[-1] ** -0.5, causal=causal, kernel_mode='hip')\n"
+        "    truth = o.attention_pullback_blocked(q, k, v, g, softmax_scale=shape[-1] ** -0.5, causal=causal, dtype=torch.float32)\n"
         "    for a, c in zip(got, truth):\n"
         "        worst = max(worst, float((a.cpu().double() - c.double()).abs().max() / c.double().abs().max()))\n"
         "print(worst); sys.exit(0 if 0.0 < worst <= 2e-2 else 1)"
