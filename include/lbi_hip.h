@@ -217,6 +217,36 @@ int lbi_attn_qkv_conv_pullback(const void* dq, const void* dk, const void* dv,
                                int64_t Dh, int interleaved, int64_t ksize, int dtype, void* stream);
 
 /*
+ * Parameter gradients of a Transformer block that are not matrix products (the others are plain GEMMs of a
+ * module's output cotangent with its cached input).  Part of TransformerLowering.parameter_vjp of the reference
+ * (backends/transformer.py:76-85; autograd version :332-355, which gets them from torch.autograd.grad).
+ * Sums run in a fixed order (per-workgroup partial sums in `workspace`, added in workgroup order): reruns are
+ * bit-identical.  Results are fp32.
+ *
+ * RMSNorm weight:  weight_grad[c] = sum over rows of g_out[row,c] * round(x_r[row,c] * rsqrt(mean_c(x_r^2) + eps)),
+ *   x_r = x rounded to `dtype` (RMSNorm.forward, reference backbones/transformer/block.py:12-23).
+ *   g_out [rows,D] in `dtype` (the weight's), x [rows,D] in `x_dtype` (= dtype, or fp32 for an fp32 residual
+ *   stream); D a multiple of 4, at most 2048.  workspace: lbi_rmsnorm_weight_grad_workspace_bytes(rows, D) bytes,
+ *   16-byte aligned.
+ */
+size_t lbi_rmsnorm_weight_grad_workspace_bytes(int64_t rows, int64_t D);
+int lbi_rmsnorm_weight_grad(const void* g_out, const void* x, float* weight_grad,
+                            void* workspace, size_t workspace_bytes,
+                            int64_t rows, int64_t D, float eps, int dtype, int x_dtype, void* stream);
+
+/*
+ * Depthwise causal convolution (reference backends/transformer.py:121-122: Conv1d(groups=C, padding=k-1),
+ * first T outputs), weight and bias gradient:
+ *   grads[c*k + j]   = sum over b, t >= k-1-j of g_out[b,t,c] * x[b, t-(k-1-j), c]      (weight [C,1,k])
+ *   grads[C*k + c]   = sum over b, t of g_out[b,t,c]                                    (bias [C])
+ *   g_out, x [B,T,C] in `dtype`; k <= 8.  workspace: lbi_causal_conv1d_weight_grad_workspace_bytes(B,T,C,k) bytes.
+ */
+size_t lbi_causal_conv1d_weight_grad_workspace_bytes(int64_t B, int64_t T, int64_t C, int64_t ksize);
+int lbi_causal_conv1d_weight_grad(const void* g_out, const void* x, float* grads,
+                                  void* workspace, size_t workspace_bytes,
+                                  int64_t B, int64_t T, int64_t C, int64_t ksize, int dtype, void* stream);
+
+/*
  * Frobenius and spectral (largest singular value) norms of N square matrices, the per-step Jacobian
  * diagnostics of the interface scan (reference backward/suffix_scan.py:105-134, which calls
  * torch.linalg.matrix_norm with ord="fro" and ord=2, a singular value decomposition per matrix).

@@ -14,7 +14,7 @@ import torch
 LIB_PATH = Path(__file__).resolve().parent / "liblbi_hip.so"
 
 LBI_F32, LBI_F16, LBI_BF16 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _DTYPE_CODES = {torch.float32: LBI_F32, torch.float16: LBI_F16, torch.bfloat16: LBI_BF16}
 
@@ -64,6 +64,16 @@ SYMBOLS = {
     "lbi_matrix_norms": (
         _c.c_int,
         [_c.c_void_p] * 4 + [_c.c_size_t, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p],
+    ),
+    "lbi_rmsnorm_weight_grad_workspace_bytes": (_c.c_size_t, [_c.c_int64, _c.c_int64]),
+    "lbi_rmsnorm_weight_grad": (
+        _c.c_int,
+        [_c.c_void_p] * 4 + [_c.c_size_t, _c.c_int64, _c.c_int64, _c.c_float, _c.c_int, _c.c_int, _c.c_void_p],
+    ),
+    "lbi_causal_conv1d_weight_grad_workspace_bytes": (_c.c_size_t, [_c.c_int64] * 4),
+    "lbi_causal_conv1d_weight_grad": (
+        _c.c_int,
+        [_c.c_void_p] * 4 + [_c.c_size_t] + [_c.c_int64] * 4 + [_c.c_int, _c.c_void_p],
     ),
 }
 

@@ -14,7 +14,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "liblbi_hip.so"
-SOURCES = ("lbi_common.hip", "lbi_scan.hip", "lbi_attn.hip", "lbi_region.hip", "lbi_norms.hip")
+SOURCES = ("lbi_common.hip", "lbi_scan.hip", "lbi_attn.hip", "lbi_region.hip", "lbi_norms.hip", "lbi_param_grads.hip")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -204,6 +204,55 @@ def attn_qkv_conv_pullback(dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor,
     return out
 
 
+#: widest RMSNorm and longest convolution filter the parameter-gradient kernels take
+NORM_GRAD_MAX_WIDTH = 2048
+CONV_GRAD_MAX_TAPS = 8
+
+
+def rmsnorm_weight_grad(g_out: torch.Tensor, x: torch.Tensor, eps: float) -> torch.Tensor:
+    """Gradient of an RMSNorm weight, fp32 ``[D]``: ``g_out [..., D]`` (in the weight dtype) summed over all rows
+    against the normalised input, with ``x [..., D]`` (weight dtype or fp32) rounded to the weight dtype first and
+    the normalised value rounded again, as the forward does (reference backbones/transformer/block.py:18-23)."""
+    _require_cuda(g_out, x)
+    width = g_out.shape[-1]
+    if x.shape[-1] != width or x.numel() != g_out.numel():
+        raise ValueError("rmsnorm_weight_grad: g_out and x must hold the same rows of the same width")
+    if x.dtype not in (g_out.dtype, torch.float32):
+        raise ValueError("rmsnorm_weight_grad: x must be in the dtype of g_out or fp32")
+    g_out, x = g_out.contiguous(), x.contiguous()
+    rows = g_out.numel() // width
+    out = torch.empty(width, device=g_out.device, dtype=torch.float32)
+    lib = _lib.load()
+    with torch.cuda.device(out.device):
+        need = int(lib.lbi_rmsnorm_weight_grad_workspace_bytes(rows, width))
+        workspace = torch.empty(max(need, 16), device=out.device, dtype=torch.uint8)
+        status = lib.lbi_rmsnorm_weight_grad(g_out.data_ptr(), x.data_ptr(), out.data_ptr(), workspace.data_ptr(),
+                                             workspace.numel(), rows, width, float(eps), _lib.dtype_code(g_out.dtype),
+                                             _lib.dtype_code(x.dtype), _stream(out))
+    _lib.check(status, "lbi_rmsnorm_weight_grad")
+    return out
+
+
+def causal_conv1d_weight_grad(g_out: torch.Tensor, x: torch.Tensor, ksize: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Weight ``[C, 1, k]`` and bias ``[C]`` gradients (fp32) of the depthwise causal convolution for
+    ``g_out, x [B, T, C]``: ``g_w[c, 0, j] = sum_{b, t} g_out[b, t, c] x[b, t - (k-1-j), c]``."""
+    _require_cuda(g_out, x)
+    if g_out.dim() != 3 or x.shape != g_out.shape or x.dtype != g_out.dtype:
+        raise ValueError("causal_conv1d_weight_grad: g_out and x must share shape [B, T, C] and dtype")
+    bsz, seqlen, channels = g_out.shape
+    g_out, x = g_out.contiguous(), x.contiguous()
+    out = torch.empty(channels * ksize + channels, device=g_out.device, dtype=torch.float32)
+    lib = _lib.load()
+    with torch.cuda.device(out.device):
+        need = int(lib.lbi_causal_conv1d_weight_grad_workspace_bytes(bsz, seqlen, channels, ksize))
+        workspace = torch.empty(max(need, 16), device=out.device, dtype=torch.uint8)
+        status = lib.lbi_causal_conv1d_weight_grad(g_out.data_ptr(), x.data_ptr(), out.data_ptr(), workspace.data_ptr(),
+                                                   workspace.numel(), bsz, seqlen, channels, ksize,
+                                                   _lib.dtype_code(g_out.dtype), _stream(out))
+    _lib.check(status, "lbi_causal_conv1d_weight_grad")
+    return out[:channels * ksize].view(channels, 1, ksize), out[channels * ksize:]
+
+
 def _apply_transposed(g: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``g @ weight`` for ``weight [out, in]``: the pullback of ``y = x weight^T``.  Issued as
     the library's ``A B^T`` form on a transposed copy of the (small) weight, which is its faster
@@ -229,6 +278,11 @@ def _norm_weight_grad(sink: dict, norm: Any, g_out: torch.Tensor, x: torch.Tenso
     the weight dtype first and the normalised value rounded again, as the forward does
     (reference backbones/transformer/block.py:18-23)."""
     wdtype = norm.weight.dtype
+    width = x.shape[-1]
+    if g_out.dtype == wdtype and x.dtype in (wdtype, torch.float32) and width % 4 == 0 and width <= NORM_GRAD_MAX_WIDTH:
+        sink[id(norm.weight)] = rmsnorm_weight_grad(g_out, x, norm.eps).to(wdtype)
+        return
+    # widths the kernel does not take: the same sum with torch operations on the device
     xf = x.to(wdtype).float()
     normed = (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + norm.eps)).to(wdtype).float()
     sink[id(norm.weight)] = (_rows(g_out).float() * _rows(normed)).sum(dim=0).to(wdtype)
@@ -237,6 +291,13 @@ def _norm_weight_grad(sink: dict, norm: Any, g_out: torch.Tensor, x: torch.Tenso
 def _conv_grads(sink: dict, conv: Any, g_out: torch.Tensor, x_pre: torch.Tensor) -> None:
     """Depthwise causal convolution: g_w[c, j] = sum_{b,t} g_out[b,t,c] x_pre[b, t + j - (k-1), c]."""
     ksize = conv.weight.shape[-1]
+    if ksize <= CONV_GRAD_MAX_TAPS and x_pre.dtype == g_out.dtype:
+        g_weight, g_bias = causal_conv1d_weight_grad(g_out[:, 0], x_pre, ksize)
+        sink[id(conv.weight)] = g_weight.to(conv.weight.dtype)
+        if getattr(conv, "bias", None) is not None:
+            sink[id(conv.bias)] = g_bias.to(conv.bias.dtype)
+        return
+    # longer filters: the same sums with torch operations on the device
     g = g_out[:, 0].float()
     x = x_pre.float()
     seqlen = g.shape[1]
@@ -406,6 +467,6 @@ def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tenso
 
 
 __all__ = [
-    "attn_heads_split", "attn_qkv_conv_pullback", "attn_qkv_pullback", "causal_conv1d_pullback", "gated_mlp_pullback",
-    "rmsnorm_pullback", "region_input_pullback_basis", "region_parameter_vjp", "rope_tables",
+    "attn_heads_split", "attn_qkv_conv_pullback", "attn_qkv_pullback", "causal_conv1d_pullback",
+    "causal_conv1d_weight_grad", "gated_mlp_pullback", "rmsnorm_pullback", "rmsnorm_weight_grad", "region_input_pullback_basis", "region_parameter_vjp", "rope_tables",
 ]

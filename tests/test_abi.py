@@ -75,6 +75,17 @@ def test_region_and_norm_entry_points_validate_on_the_host():
     assert lib.lbi_matrix_norms(one, one, one, None, 0, 4, 256, f32, None) == -4
     assert b"workspace" in lib.lbi_last_error()
     assert lib.lbi_matrix_norms(None, None, None, None, 0, 0, 16, f32, None) == 0
+    # parameter gradients that are not matrix products
+    assert lib.lbi_rmsnorm_weight_grad_workspace_bytes(8192, 768) == 256 * 768 * 4
+    assert lib.lbi_rmsnorm_weight_grad_workspace_bytes(10, 768) == 10 * 768 * 4
+    assert lib.lbi_rmsnorm_weight_grad(one, one, one, one, 1 << 30, 4, 6, 1e-5, f32, f32, None) == -2
+    assert b"multiple of 4" in lib.lbi_last_error()
+    assert lib.lbi_rmsnorm_weight_grad(one, one, one, None, 0, 4, 8, 1e-5, f32, f32, None) == -4
+    assert lib.lbi_rmsnorm_weight_grad(one, one, one, one, 1 << 30, 4, 8, 1e-5, f32, _lib.LBI_F16, None) == -2
+    assert lib.lbi_causal_conv1d_weight_grad_workspace_bytes(8, 1024, 2304, 4) == 8 * 16 * (2304 * 5) * 4
+    assert lib.lbi_causal_conv1d_weight_grad(one, one, one, one, 1 << 30, 1, 4, 8, 9, f32, None) == -2
+    assert b"above 8" in lib.lbi_last_error()
+    assert lib.lbi_causal_conv1d_weight_grad(one, one, one, None, 0, 1, 4, 8, 4, f32, None) == -4
     # attention: short 16-bit sequences at head dim 64 run as one launch and need no workspace
     f16 = _lib.LBI_F16
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f16) == 0

@@ -140,6 +140,66 @@ def test_causal_conv1d_pullback(dtype, channels, ksize, seqlen, device):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows_shape,dim,wide_x", [((2, 5), 32, True), ((3, 1, 7), 36, False), ((1, 300), 768, True),
+                                                  ((4, 130), 2048, False), ((1, 1), 4, True)])
+def test_rmsnorm_weight_grad(dtype, rows_shape, dim, wide_x, device):
+    """Autograd of the norm's forward (input rounded to the weight dtype, normalised value rounded again, reference
+    backbones/transformer/block.py:18-23) with respect to the weight, in fp64 on the rounded values."""
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(dim + len(rows_shape))
+    g = torch.randn(*rows_shape, dim).to(dtype)
+    x = torch.randn(*rows_shape, dim) * 1.7
+    x = x if wide_x else x.to(dtype)
+    got = region.rmsnorm_weight_grad(g.to(device), x.to(device), 1e-5)
+    assert got.dtype == torch.float32 and got.shape == (dim,)
+    xr = x.to(dtype).float()
+    normed = (xr * torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + 1e-5)).to(dtype)
+    want = (g.double() * normed.double()).reshape(-1, dim).sum(0)
+    # the normalised value is rounded to the storage type before the sum: a last-place difference of the fp32
+    # rsqrt can move single elements by one storage ulp
+    assert _max_rel(got.cpu(), want) <= (2e-5 if dtype == torch.float32 else 2e-3)
+    again = region.rmsnorm_weight_grad(g.to(device), x.to(device), 1e-5)
+    assert torch.equal(got, again)
+
+
+def test_rmsnorm_weight_grad_contract(device):
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    g = torch.zeros(2, 3, 8, device=device)
+    with pytest.raises(ValueError):
+        region.rmsnorm_weight_grad(g, torch.zeros(2, 3, 4, device=device), 1e-5)
+    with pytest.raises(ValueError):
+        region.rmsnorm_weight_grad(g.half(), torch.zeros(2, 3, 8, device=device, dtype=torch.bfloat16), 1e-5)
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        region.rmsnorm_weight_grad(torch.zeros(2, 6, device=device), torch.zeros(2, 6, device=device), 1e-5)
+    empty = region.rmsnorm_weight_grad(torch.zeros(0, 8, device=device), torch.zeros(0, 8, device=device), 1e-5)
+    assert torch.equal(empty.cpu(), torch.zeros(8))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bsz,seqlen,channels,ksize", [(2, 10, 8, 4), (3, 2, 6, 3), (1, 4, 5, 1), (2, 130, 2304, 4),
+                                                      (1, 70, 12, 8), (2, 3, 7, 5)])
+def test_causal_conv1d_weight_grad(dtype, bsz, seqlen, channels, ksize, device):
+    """Autograd of Conv1d(groups=C, padding=k-1) cut to the first T outputs (reference
+    backends/transformer.py:121-122) with respect to weight and bias, in fp64 on the stored values."""
+    from latent_bounded_interfaces_amd.hip.transformer import region
+
+    torch.manual_seed(channels + ksize + seqlen)
+    g = torch.randn(bsz, seqlen, channels).to(dtype)
+    x = torch.randn(bsz, seqlen, channels).to(dtype)
+    g_w, g_b = region.causal_conv1d_weight_grad(g.to(device), x.to(device), ksize)
+    assert g_w.shape == (channels, 1, ksize) and g_b.shape == (channels,) and g_w.dtype == torch.float32
+    w = torch.zeros(channels, 1, ksize, dtype=torch.float64, requires_grad=True)
+    b = torch.zeros(channels, dtype=torch.float64, requires_grad=True)
+    y = F.conv1d(x.double().transpose(1, 2), w, b, padding=ksize - 1, groups=channels)[..., :seqlen].transpose(1, 2)
+    want_w, want_b = torch.autograd.grad(y, (w, b), grad_outputs=g.double())
+    assert _max_rel(g_w.cpu(), want_w) <= 2e-5 and _max_rel(g_b.cpu(), want_b) <= 2e-5
+    again = region.causal_conv1d_weight_grad(g.to(device), x.to(device), ksize)
+    assert torch.equal(g_w, again[0]) and torch.equal(g_b, again[1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,head_dim,interleaved,ksize,seqlen",
                          [(4, 2, 8, False, 4, 19), (4, 4, 8, True, 3, 8), (3, 1, 6, False, 4, 5), (3, 1, 2, True, 1, 9),
                           (12, 4, 64, False, 4, 33), (2, 1, 64, True, 7, 12), (2, 2, 16, False, 8, 3)])
