@@ -253,10 +253,16 @@ def causal_conv1d_weight_grad(g_out: torch.Tensor, x: torch.Tensor, ksize: int) 
     return out[:channels * ksize].view(channels, 1, ksize), out[channels * ksize:]
 
 
+#: rows below which the transposed copy of the weight costs more than the faster product form gains
+_TRANSPOSED_COPY_MIN_ROWS = 65536
+
+
 def _apply_transposed(g: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """``g @ weight`` for ``weight [out, in]``: the pullback of ``y = x weight^T``.  Issued as
-    the library's ``A B^T`` form on a transposed copy of the (small) weight, which is its faster
-    path for these tall products."""
+    """``g @ weight`` for ``weight [out, in]``: the pullback of ``y = x weight^T``.  For tall ``g`` it is issued as
+    the library's ``A B^T`` form on a transposed copy of the (small) weight, which is its faster path for these
+    products; for few rows (the single direction of a parameter VJP) the copy is not worth it."""
+    if g.numel() // g.shape[-1] < _TRANSPOSED_COPY_MIN_ROWS:
+        return torch.matmul(g, weight)
     return torch.nn.functional.linear(g, weight.t().contiguous())
 
 
