@@ -538,6 +538,79 @@ __global__ __launch_bounds__(512) void cotangent256_kernel(const float* __restri
     }
 }
 
+// The same chain for 16-bit storage: a row is 512 bytes, so a load instruction covers two rows (lane half = row,
+// 8 elements per lane) and a wave's 32 rows are 16 registers in flight; the 16 partial sums of a lane are folded
+// across the 32 lanes of its half.
+template <typename Tin>
+__global__ __launch_bounds__(512) void cotangent256_half_kernel(const Tin* __restrict__ mats,
+                                                                const float* __restrict__ g, float* __restrict__ out,
+                                                                int K) {
+    constexpr int D = 256;
+    typedef unsigned int raw4 __attribute__((ext_vector_type(4)));
+    __shared__ __align__(16) float vbuf[2][D];
+    const int b = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, sub = lane >> 5, piece = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const Tin* mats_b = mats + (size_t)b * K * D * D;
+    float* out_b = out + (size_t)b * (K + 1) * D;
+    if (tid < D) {
+        const float val = g[(size_t)b * D + tid];
+        vbuf[0][tid] = val;
+        out_b[(size_t)K * D + tid] = val;
+    }
+    if (K == 0) return;
+    // Row wave + 8 * (2 i + sub) of matrix r, elements 8 * piece .. 8 * piece + 7.
+    auto load_row = [&](int r, int i) {
+        return *reinterpret_cast<const raw4*>(mats_b + (size_t)r * D * D + (size_t)(wave + 8 * (2 * i + sub)) * D + 8 * piece);
+    };
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    raw4 buf[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) buf[i] = load_row(K - 1, i);
+    lds_barrier();
+    int cur = 0;
+    for (int r = K - 1; r >= 0; --r) {
+        const f32x4 v_lo = *reinterpret_cast<const f32x4*>(&vbuf[cur][8 * piece]);
+        const f32x4 v_hi = *reinterpret_cast<const f32x4*>(&vbuf[cur][8 * piece + 4]);
+        const int r_next = r > 0 ? r - 1 : 0;  // a harmless re-read at the end
+        float vals[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const Tin* e = reinterpret_cast<const Tin*>(&buf[i]);
+            float acc = to_f32(e[0]) * v_lo[0];
+#pragma unroll
+            for (int q = 1; q < 4; ++q) acc = fmaf(to_f32(e[q]), v_lo[q], acc);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc = fmaf(to_f32(e[4 + q]), v_hi[q], acc);
+            vals[i] = acc;
+            buf[i] = load_row(r_next, i);
+            __builtin_amdgcn_sched_barrier(0);  // keep the refill next to the use
+        }
+        // Halving butterfly inside each 32-lane half: lane `piece` ends with value index piece >> 1.
+        auto stage = [&](auto half_tag) {
+            constexpr int HALF = decltype(half_tag)::value;
+            const bool up = (lane & (2 * HALF)) != 0;
+            float got[HALF];
+#pragma unroll
+            for (int i = 0; i < HALF; ++i) got[i] = __shfl_xor(up ? vals[i] : vals[i + HALF], 2 * HALF, 64);
+#pragma unroll
+            for (int i = 0; i < HALF; ++i) vals[i] = (up ? vals[i + HALF] : vals[i]) + got[i];
+        };
+        stage(std::integral_constant<int, 8>{});
+        stage(std::integral_constant<int, 4>{});
+        stage(std::integral_constant<int, 2>{});
+        stage(std::integral_constant<int, 1>{});
+        const float total = vals[0] + __shfl_xor(vals[0], 1, 64);
+        if ((lane & 1) == 0) {
+            const int row = wave + 8 * (2 * (piece >> 1) + sub);
+            vbuf[cur ^ 1][row] = total;
+            out_b[(size_t)r * D + row] = total;
+        }
+        lds_barrier();
+        cur ^= 1;
+    }
+}
+
 template <typename Tin, int D, int RT, int CB, bool COT>
 int launch_mfma_cot(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
     constexpr int NW = D / RT;
@@ -640,6 +713,12 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
     const int threads = d >= 128 ? 512 : (d >= 32 ? 256 : 64);
     if (d == 256 && std::is_same<Tin, float>::value) {
         hipLaunchKernelGGL(cotangent256_kernel, dim3(B), dim3(512), 0, stream, static_cast<const float*>(mats),
+                           static_cast<const float*>(g), static_cast<float*>(out), K);
+        LBI_HIP_CHECK(hipGetLastError());
+        return LBI_OK;
+    }
+    if constexpr (sizeof(Tin) == 2) if (d == 256) {
+        hipLaunchKernelGGL(cotangent256_half_kernel<Tin>, dim3(B), dim3(512), 0, stream, static_cast<const Tin*>(mats),
                            static_cast<const float*>(g), static_cast<float*>(out), K);
         LBI_HIP_CHECK(hipGetLastError());
         return LBI_OK;
