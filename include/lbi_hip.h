@@ -256,7 +256,8 @@ int lbi_causal_conv1d_weight_grad(const void* g_out, const void* x, float* grads
  * No decomposition: the top eigenvalue of A^T A comes from repeated squaring with the trace divided
  * out, at most 24 squarings, which bounds the relative error by 2^-25 log(d) plus fp32 rounding for
  * any spectrum.  `workspace` must hold lbi_matrix_norms_workspace_bytes(N, d) bytes (0 for d <= 88,
- * whose buffers fit in LDS), 16-byte aligned.  d <= 2048.
+ * whose buffers fit in LDS; larger matrices run their products on the fp32 matrix cores out of the
+ * workspace), 16-byte aligned.  d <= 2048.
  */
 size_t lbi_matrix_norms_workspace_bytes(int64_t N, int64_t d);
 int lbi_matrix_norms(const void* mats, float* spectral, float* frobenius,

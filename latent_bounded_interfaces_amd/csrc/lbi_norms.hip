@@ -10,7 +10,10 @@
 // rounding whatever the spectrum; well-separated spectra stop after a handful of squarings.
 //
 // One workgroup per matrix (grid-stride over the batch).  The two d x d fp32 buffers live in LDS when they
-// fit in 64 KB, otherwise in a per-workgroup slice of the caller's workspace (L2 resident).
+// fit in 64 KB (d <= 88: scalar products), otherwise in a per-workgroup slice of the caller's workspace (L2
+// resident), padded to a multiple of 32 so that the products run on the fp32 matrix cores
+// (v_mfma_f32_32x32x2_f32): the Gram matrix is then X X^T, which has the same top eigenvalue as X^T X, both
+// operands are row strips, and only the tiles on and above the diagonal are formed and mirrored.
 #include "lbi_common.h"
 
 namespace lbi {
@@ -20,8 +23,12 @@ constexpr int THREADS = 256;
 constexpr int MAX_SQUARINGS = 24;
 constexpr int LDS_LIMIT_BYTES = 64 * 1024;
 
-inline int padded(int d) { return (d + 3) & ~3; }
 inline bool fits_lds(int ld) { return 2ll * ld * ld * 4 <= LDS_LIMIT_BYTES; }
+// leading dimension of the buffers: a multiple of 4 in LDS, of 32 (matrix-core tiles) in the workspace
+inline int padded(int d) {
+    const int ld4 = (d + 3) & ~3;
+    return fits_lds(ld4) ? ld4 : (d + 31) & ~31;
+}
 inline int grid_for(long long n, int ld) {
     const long long cap = ld <= 256 ? 1024 : 256;
     return (int)(n < cap ? n : cap);
@@ -65,6 +72,42 @@ __device__ __forceinline__ void gram(const float* X, float* H, int ld) {
     }
 }
 
+// H = X X^T for ld x ld row-major X, ld a multiple of 32, on the fp32 matrix cores (for symmetric X this is X^2).
+// Tile (ti, tj), ti <= tj, is sum_k X[32 ti + m][k] X[32 tj + n][k]: both operands are 16-byte pieces of rows (a lane
+// of half h takes k = 8 q + 4 h + e for the e-th product of piece q, the same on both sides).  The tiles on and
+// above the diagonal are dealt to the four waves in turn; each is written twice, so H is exactly symmetric.
+// `scale` multiplies the result (the normalisation of X folded into the product: (cX)(cX)^T = c^2 X X^T).
+__device__ __forceinline__ void gram_mfma(const float* X, float* H, int ld, float scale) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m = lane & 31, h = lane >> 5;
+    const int nt = ld >> 5;
+    int turn = 0;
+    for (int ti = 0; ti < nt; ++ti)
+        for (int tj = ti; tj < nt; ++tj, ++turn) {
+            if ((turn & 3) != wave) continue;
+            const float* a_row = X + (long long)(32 * ti + m) * ld + 4 * h;
+            const float* b_row = X + (long long)(32 * tj + m) * ld + 4 * h;
+            f32x16 acc;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+#pragma unroll 4
+            for (int q = 0; q < ld / 8; ++q) {
+                const f32x4 a = *reinterpret_cast<const f32x4*>(a_row + 8 * q);
+                const f32x4 b = *reinterpret_cast<const f32x4*>(b_row + 8 * q);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e] * scale, b[e], acc, 0, 0, 0);
+            }
+            // register 4 g + e of lane (m, h) is row 8 g + 4 h + e, column m of the tile
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) H[(long long)(32 * ti + 8 * g + 4 * h + e) * ld + 32 * tj + m] = acc[4 * g + e];
+                if (ti != tj)
+                    *reinterpret_cast<f32x4*>(H + (long long)(32 * tj + m) * ld + 32 * ti + 8 * g + 4 * h) =
+                        f32x4{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+            }
+        }
+}
+
 template <typename T>
 __global__ __launch_bounds__(THREADS) void matrix_norms_kernel(const T* __restrict__ mats, float* __restrict__ spectral,
                                                                float* __restrict__ frobenius, float* scratch, long long n,
@@ -100,7 +143,8 @@ __global__ __launch_bounds__(THREADS) void matrix_norms_kernel(const T* __restri
 
         float* x = buf0;
         float* h = buf1;
-        gram(x, h, ld);
+        if (use_lds) gram(x, h, ld);
+        else gram_mfma(x, h, ld, 1.0f);
         float log_lambda = 0.0f, weight = 1.0f;
         for (int step = 0;; ++step) {
             float tr = 0.0f;  // block_sum's first barrier publishes h
@@ -109,10 +153,18 @@ __global__ __launch_bounds__(THREADS) void matrix_norms_kernel(const T* __restri
             tr = block_sum(tr, red);
             const float inv_tr = 1.0f / tr;
             float q = 0.0f;
-            for (int idx = threadIdx.x; idx < (int)plane; idx += THREADS) {
-                const float v = h[idx] * inv_tr;
-                h[idx] = v;
-                q = fmaf(v, v, q);
+            if (use_lds) {
+                for (int idx = threadIdx.x; idx < (int)plane; idx += THREADS) {
+                    const float v = h[idx] * inv_tr;
+                    h[idx] = v;
+                    q = fmaf(v, v, q);
+                }
+            } else {  // h stays as it is: the next product takes the factor, this pass only reads
+                for (int idx = 4 * threadIdx.x; idx < (int)plane; idx += 4 * THREADS) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(h + idx);
+                    q = fmaf(v[0], v[0], fmaf(v[1], v[1], fmaf(v[2], v[2], fmaf(v[3], v[3], q))));
+                }
+                q *= inv_tr * inv_tr;
             }
             q = block_sum(q, red);
             log_lambda += weight * logf(tr);
@@ -124,7 +176,8 @@ __global__ __launch_bounds__(THREADS) void matrix_norms_kernel(const T* __restri
             float* t = x;
             x = h;
             h = t;
-            gram(x, h, ld);
+            if (use_lds) gram(x, h, ld);
+            else gram_mfma(x, h, ld, inv_tr * inv_tr);
             weight *= 0.5f;
         }
         if (threadIdx.x == 0) {

@@ -69,7 +69,7 @@ def test_region_and_norm_entry_points_validate_on_the_host():
     # spectral / Frobenius norms: LDS-resident sizes need no workspace, larger ones two planes per workgroup
     assert lib.lbi_matrix_norms_workspace_bytes(10, 64) == 0
     assert lib.lbi_matrix_norms_workspace_bytes(10, 88) == 0
-    assert lib.lbi_matrix_norms_workspace_bytes(10, 90) == 10 * 2 * 92 * 92 * 4
+    assert lib.lbi_matrix_norms_workspace_bytes(10, 90) == 10 * 2 * 96 * 96 * 4
     assert lib.lbi_matrix_norms_workspace_bytes(5000, 256) == 1024 * 2 * 256 * 256 * 4
     assert lib.lbi_matrix_norms(one, one, one, None, 0, 4, 0, f32, None) == -1
     assert lib.lbi_matrix_norms(one, one, one, None, 0, 4, 256, f32, None) == -4
