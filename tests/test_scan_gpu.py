@@ -101,7 +101,7 @@ def test_permutations_are_exact(device):
 
 
 @pytest.mark.parametrize("shape", [(1, 0, 3), (2, 1, 8), (3, 5, 7), (4, 8, 32), (2, 6, 64), (3, 9, 128),
-                                   (5, 12, 256), (2, 3, 100), (2, 4, 260)])
+                                   (5, 12, 256), (2, 3, 100), (2, 4, 260), (2, 0, 256), (3, 1, 256), (1, 2, 256)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_cotangent_chain_matches_oracle(shape, dtype, device):
     from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents
