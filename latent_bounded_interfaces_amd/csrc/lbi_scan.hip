@@ -681,6 +681,12 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
         // the chip enough workgroups, and the blocks of an element run side by side and share the matrices in L2.
         // With many, they drift apart and fetch them again (measured 1.7x / 2.4x the input bytes at d = 64 / 128),
         // so one workgroup then takes all columns.
+        case 512: {
+            // 16 column blocks of 32 per batch element, 8 waves of 64 rows.  The fused form would spill, so the
+            // cotangent chain, if asked for, runs as its own kernel behind the matrices.
+            if (int rc = launch_mfma<Tin, 512, 64, 32>(mats, out, nullptr, nullptr, B, K, stream)) return rc;
+            return cot ? launch_cotangent<Tin>(mats, g, cot, B, K, d, stream) : LBI_OK;
+        }
         case 128:
             if (B >= kWideBlockBatch) return launch_mfma<Tin, 128, 32, 128>(mats, out, g, cot, B, K, stream);
             return launch_mfma<Tin, 128, 32, 32>(mats, out, g, cot, B, K, stream);

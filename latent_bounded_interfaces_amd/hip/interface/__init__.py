@@ -30,7 +30,7 @@ def _validate(mats: torch.Tensor) -> tuple[int, int, int]:
 
 
 #: interface widths the matrix-core scan kernels are built for
-_MFMA_WIDTHS = (32, 64, 128, 256)
+_MFMA_WIDTHS = (32, 64, 128, 256, 512)
 
 
 def _padded_width(rank: int) -> int:

@@ -19,7 +19,8 @@ SHAPES = [
     (1, 0, 1), (1, 1, 1), (1, 1, 4), (2, 3, 5), (2, 4, 8), (4, 8, 16), (1, 16, 64),
     (1, 2, 16), (2, 4, 32), (2, 8, 64), (1, 16, 128), (1, 8, 256),
     (4, 8, 32), (3, 5, 32), (9, 7, 64), (5, 3, 128), (3, 5, 256), (2, 6, 48), (2, 3, 33), (1, 4, 100),
-    (1, 3, 300), (2, 5, 12),  # widths the scalar kernel still runs: past the largest matrix-core width, and tiny
+    (1, 3, 300), (2, 3, 512), (1, 2, 384),  # the widest matrix-core kernel, directly and through padding
+    (1, 2, 520), (2, 5, 12),  # widths the scalar kernel still runs: past the largest matrix-core width, and tiny
     (17, 2, 256), (1, 1, 256), (2, 0, 32),
 ]
 
@@ -121,7 +122,7 @@ def test_cotangent_chain_matches_oracle(shape, dtype, device):
 
 
 @pytest.mark.parametrize("shape", [(1, 0, 3), (2, 1, 8), (3, 5, 7), (4, 8, 32), (2, 6, 64), (3, 9, 128), (5, 12, 256),
-                                   (9, 1, 256), (2, 2, 32), (2, 3, 100), (1, 1, 64)])
+                                   (9, 1, 256), (2, 2, 32), (2, 3, 100), (1, 1, 64), (2, 3, 512), (1, 2, 300)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_fused_scan_and_cotangents(shape, dtype, device):
     """One pass giving both results equals the two separate entry points (bit-exact for the
