@@ -101,7 +101,7 @@ int lbi_suffix_cotangents(const void* mats, const void* g, void* out,
  * taken from the caller).  `workspace` must hold at least
  * lbi_attn_pullback_workspace_bytes(...) bytes of device memory, 256-byte
  * aligned; its contents on entry are ignored.  That size is 0 for short
- * sequences (16-bit storage, T a multiple of 32, up to 256 at Dh = 64 and up
+ * sequences (16-bit storage, any T up to 256 at Dh = 64 and up
  * to 128 at Dh = 128), which run as a single launch; `workspace` may then be
  * null.  Replaces
  * attention_input_pullback_basis_simple / _mma_p1 / _mma_pblock4 of the

@@ -1,5 +1,5 @@
-// Attention input-pullback for short sequences in one launch (fp16 / bf16 storage; T a multiple of 32, up to
-// 256 at head dim 64 and up to 128 at head dim 128).
+// Attention input-pullback for short sequences in one launch (fp16 / bf16 storage; any T up to 256 at head dim
+// 64 and up to 128 at head dim 128).
 //
 // At these sizes a call is bound by launch and pipeline-fill latency, not by arithmetic, so one
 // workgroup does everything for one (b, h, direction): Q, K, V and d_out_p (T x Dh each) are
@@ -11,6 +11,8 @@
 //   pass 2, per owned tile of 32 keys (lanes = keys, registers = queries, as in the dK/dV kernel):
 //     S = Q K^T, P = exp2(S c - lse), dP = dO V^T, dS = P (dP - delta),
 //     dV = P^T dO, dK = scale dS^T Q
+// A length that is no multiple of 32 fills its last tile with zero rows: as keys they are masked out (the causal
+// mask already does that), as queries they carry a zero cotangent and add nothing; their outputs are not stored.
 // Every output tile has one owner and every sum a fixed order: reruns are bit-identical.
 #pragma once
 
@@ -29,7 +31,7 @@ static_assert(lds_bytes<64, 8>() <= 160 * 1024 && lds_bytes<128, 4>() <= 160 * 1
 
 inline int max_seq(int dh) { return dh == 64 ? 256 : (dh == 128 ? 128 : 0); }
 inline bool supports(int T_len, int dh, int dtype) {
-    return (dtype == LBI_F16 || dtype == LBI_BF16) && T_len >= 32 && T_len <= max_seq(dh) && T_len % 32 == 0;
+    return (dtype == LBI_F16 || dtype == LBI_BF16) && T_len >= 1 && T_len <= max_seq(dh);
 }
 
 // Four values of one output row (consecutive head-dim elements), scaled, as 8 bytes.
@@ -58,7 +60,7 @@ __global__ __launch_bounds__(256, (DH == 64 && MAX_TILES == 4) ? 2 : 1) void sma
 
     int bh, p;
     if (!map_block(P, n_bh, bh, p)) return;
-    const int nt = T_len / 32;  // 1 .. MAX_TILES
+    const int nt = (T_len + 31) / 32;  // 1 .. MAX_TILES; the last tile may be partly past the end
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int b = bh / H, hh = bh - b * H;
@@ -67,14 +69,24 @@ __global__ __launch_bounds__(256, (DH == 64 && MAX_TILES == 4) ? 2 : 1) void sma
     const float sc2 = scale * LOG2E;
 
     {
+        // rows past the end of the sequence (last tile of a ragged length) are zero
+        auto fetch = [&](TileLoader<DH>& ld, const T* src, int row0) __attribute__((always_inline)) {
+            constexpr int CPR = DH / 8;
+#pragma unroll
+            for (int u = 0; u < TileLoader<DH>::N; ++u) {
+                const int id = tid + 256 * u;
+                const int r = row0 + id / CPR, c = id % CPR;
+                ld.regs[u] = r < T_len ? *reinterpret_cast<const u32x4*>(src + (size_t)r * DH + c * 8) : u32x4{0u, 0u, 0u, 0u};
+            }
+        };
         TileLoader<DH> lq[MAX_TILES], lk[MAX_TILES], lv[MAX_TILES], lg[MAX_TILES];
 #pragma unroll
         for (int t = 0; t < MAX_TILES; ++t)
             if (t < nt) {
-                lq[t].fetch(q + base, 32 * t, tid);
-                lk[t].fetch(k + base, 32 * t, tid);
-                lv[t].fetch(v + base, 32 * t, tid);
-                lg[t].fetch(d_out + gbase, 32 * t, tid);
+                fetch(lq[t], q + base, 32 * t);
+                fetch(lk[t], k + base, 32 * t);
+                fetch(lv[t], v + base, 32 * t);
+                fetch(lg[t], d_out + gbase, 32 * t);
             }
 #pragma unroll
         for (int t = 0; t < MAX_TILES; ++t)
@@ -111,10 +123,12 @@ __global__ __launch_bounds__(256, (DH == 64 && MAX_TILES == 4) ? 2 : 1) void sma
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) dp[jt] = Mma<T>::mma(frag_nat<DH>(v_lds + jt * TILE_BYTES, m, h, ks), gf[ks], dp[jt]);
                 const bool diag = CAUSAL && jt == qt;
+                const int keys_left = T_len - 32 * jt;  // < 32 only in a ragged last tile
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     float x = s[jt][r] * sc2;
                     if (diag && c_row(r, h) > m) x = -INFINITY;  // key after the query
+                    if (!CAUSAL && c_row(r, h) >= keys_left) x = -INFINITY;  // key past the end
                     s[jt][r] = x;
                     row_max = fmaxf(row_max, x);
                 }
@@ -160,11 +174,13 @@ __global__ __launch_bounds__(256, (DH == 64 && MAX_TILES == 4) ? 2 : 1) void sma
                         dq_t[nd] = Mma<T>::mma(frag_tr<DH>(k_lds + jt * TILE_BYTES, lane, 16 * kk, 32 * nd), ds_frag, dq_t[nd]);
                 }
             }
-        T* dq_row = dq + gbase + (size_t)(32 * qt + m) * DH;
+        if (32 * qt + m < T_len) {
+            T* dq_row = dq + gbase + (size_t)(32 * qt + m) * DH;
 #pragma unroll
-        for (int nd = 0; nd < ND; ++nd)
+            for (int nd = 0; nd < ND; ++nd)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) store4<T>(dq_row + 32 * nd + 8 * g + 4 * h, dq_t[nd], g, scale);
+                for (int g = 0; g < 4; ++g) store4<T>(dq_row + 32 * nd + 8 * g + 4 * h, dq_t[nd], g, scale);
+        }
         if (h == 0) {
             lse_lds[32 * qt + m] = row_max + log2f(row_sum);
             delta_lds[32 * qt + m] = delta;
@@ -224,15 +240,17 @@ __global__ __launch_bounds__(256, (DH == 64 && MAX_TILES == 4) ? 2 : 1) void sma
                 }
             }
         }
-        T* dk_row = dk + gbase + (size_t)(32 * kt + m) * DH;
-        T* dv_row = dv + gbase + (size_t)(32 * kt + m) * DH;
+        if (32 * kt + m < T_len) {
+            T* dk_row = dk + gbase + (size_t)(32 * kt + m) * DH;
+            T* dv_row = dv + gbase + (size_t)(32 * kt + m) * DH;
 #pragma unroll
-        for (int nd = 0; nd < ND; ++nd)
+            for (int nd = 0; nd < ND; ++nd)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                store4<T>(dk_row + 32 * nd + 8 * g + 4 * h, dk_t[nd], g, scale);
-                store4<T>(dv_row + 32 * nd + 8 * g + 4 * h, dv_t[nd], g, 1.0f);
-            }
+                for (int g = 0; g < 4; ++g) {
+                    store4<T>(dk_row + 32 * nd + 8 * g + 4 * h, dk_t[nd], g, scale);
+                    store4<T>(dv_row + 32 * nd + 8 * g + 4 * h, dv_t[nd], g, 1.0f);
+                }
+        }
     }
 }
 

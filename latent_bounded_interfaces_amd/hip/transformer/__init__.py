@@ -32,7 +32,7 @@ _MODE_BASIS_LIMIT = {
 # what the matrix-core kernels take (the generic kernels take any length and head dim up to 256)
 _MFMA_SEQ_MULTIPLE = 64
 _MFMA_HEAD_DIMS = (64, 128)
-# longest sequence the single-launch kernel takes, by head dim (any multiple of 32 up to it)
+# longest sequence the single-launch kernel takes, by head dim (any length up to it)
 _SINGLE_LAUNCH_MAX_SEQ = {64: 256, 128: 128}
 
 
@@ -83,17 +83,17 @@ def attention_input_pullback_basis(
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     d_out = output_cotangent_basis.contiguous()
     bsz, heads, seqlen, head_dim = q.shape
-    if q.dtype in (torch.float16, torch.bfloat16) and d_out.numel() and seqlen > _MFMA_SEQ_MULTIPLE // 2:
-        # The matrix-core kernels take head dims 64 and 128 and sequence lengths that are multiples of 64 (of 32 for
-        # short sequences); everything else runs on the generic kernels, at a small fraction of their speed.  Two paddings are exact:
+    wide_dim = next((w for w in _MFMA_HEAD_DIMS if w >= head_dim), head_dim)
+    single_launch = seqlen <= _SINGLE_LAUNCH_MAX_SEQ.get(wide_dim, 0)
+    if q.dtype in (torch.float16, torch.bfloat16) and d_out.numel() and (single_launch or seqlen > _MFMA_SEQ_MULTIPLE // 2):
+        # The matrix-core kernels take head dims 64 and 128 and sequence lengths that are multiples of 64 (short
+        # sequences, which run as a single launch, any length); everything else runs on the generic kernels, at a
+        # small fraction of their speed.  Two paddings are exact:
         # * zero columns appended to the head dim add nothing to any dot product (the scale is passed explicitly)
         #   and receive zero cotangents;
         # * under the causal mask, zero rows appended after the sequence are invisible to every real query, and as
         #   queries they carry a zero cotangent, so they add nothing to dK or dV.
-        wide_dim = next((w for w in _MFMA_HEAD_DIMS if w >= head_dim), head_dim)
-        # short sequences (up to 256 positions at head dim 64, 128 at head dim 128): the single-launch kernel takes
-        # multiples of 32
-        multiple = 32 if seqlen <= _SINGLE_LAUNCH_MAX_SEQ.get(wide_dim, 0) else _MFMA_SEQ_MULTIPLE
+        multiple = 1 if single_launch else _MFMA_SEQ_MULTIPLE
         ragged = seqlen % multiple != 0
         long_seq = seqlen + (multiple - seqlen % multiple) if (ragged and causal) else seqlen
         if (wide_dim != head_dim or long_seq != seqlen) and long_seq % multiple == 0 \

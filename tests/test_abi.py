@@ -90,6 +90,7 @@ def test_region_and_norm_entry_points_validate_on_the_host():
     f16 = _lib.LBI_F16
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f16) == 0
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 256, 64, 4, f16) == 0
+    assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 77, 64, 4, f16) == 0
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 128, 4, f16) == 0
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 320, 64, 4, f16) == 4 * (64 * 320 + 256 * 320 + 64 * 320 * 64)
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f32) > 0

@@ -81,10 +81,13 @@ LOWP_CASES = [
     # head dims below 128 that are not 64: zero-padded onto the matrix-core kernels (with the length, if causal)
     (24, (1, 2, 128, 32), 3), (25, (2, 1, 192, 96), 2), (26, (1, 2, 70, 80), 2), (27, (1, 1, 64, 8), 1),
     (28, (1, 1, 128, 160), 2),  # past 128: generic kernels
-    # lengths that are multiples of 32, up to 256 at head dim 64 and 128 at head dim 128: the single-launch kernel
+    # lengths up to 256 at head dim 64 and up to 128 at head dim 128: the single-launch kernel
     # (so are 11, 12, 13, 16, 17, 19 above and, once padded, the causal runs of 21, 23, 24, 27)
     (29, (1, 2, 32, 64), 3), (30, (3, 1, 128, 64), 1), (31, (2, 3, 96, 64), 5), (32, (1, 2, 160, 64), 2),
     (33, (2, 1, 64, 128), 3), (34, (1, 1, 96, 128), 2), (35, (1, 2, 224, 64), 1), (36, (2, 2, 256, 64), 4),
+    # the same kernel at lengths that are no multiple of 32 (zero rows in the last tile, keys past the end masked)
+    (37, (1, 2, 1, 64), 2), (38, (2, 1, 255, 64), 3), (39, (1, 2, 127, 128), 2), (40, (1, 1, 31, 64), 1),
+    (41, (2, 2, 129, 64), 2), (42, (1, 1, 5, 128), 3),
 ]
 
 
