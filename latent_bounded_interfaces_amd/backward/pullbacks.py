@@ -22,6 +22,7 @@ run again.
 """
 from __future__ import annotations
 
+import weakref
 from typing import Any
 
 import torch
@@ -40,25 +41,41 @@ class StructuredInterfacePullbackProvider:
             raise ValueError("position_constant_update must be one of: verify_once, verify, off")
         self.basis_chunk = int(basis_chunk)
         self.position_constant_update = position_constant_update
-        self._constant_over_positions: dict[type, bool] = {}
+        # (interface instance, region length) -> True once a non-zero cotangent was seen to be constant
+        self._constant_over_positions: "weakref.WeakKeyDictionary[Any, dict[int, bool]]" = weakref.WeakKeyDictionary()
 
     def _region_output_cotangent(self, interface: Any, g_region_output: torch.Tensor) -> torch.Tensor:
         """An interface that pools the region output with a mean over positions sends the same cotangent to
         every position (reference interfaces/vector_mlp.py:111-116 materialises it as a dense [B,P,T,D]
         tensor).  When that holds the tensor is handed on as a stride-0 view of its first position, which lets
-        the region pullback run the last block's first product on one row per direction.  Whether it holds is
-        a property of the interface class: it is checked on the device (one host synchronisation) the first
-        time a class is seen (``verify_once``), on every call (``verify``), or never used (``off``)."""
+        the region pullback run the last block's first product on one row per direction.
+
+        An interface may declare the property (attribute ``region_output_cotangent_constant_over_positions``:
+        True / False); otherwise it is checked on the device (one host synchronisation): on every call
+        (``verify``), or until a call has shown it for this interface object and this region length with a
+        cotangent that is not all zero (``verify_once``: an all-zero cotangent, e.g. from a zero-initialised gate,
+        is constant trivially and proves nothing about later steps).  A negative finding is never cached."""
         if self.position_constant_update == "off" or g_region_output.dim() != 4 or g_region_output.shape[2] <= 1:
             return g_region_output
         if g_region_output.stride(2) == 0:
             return g_region_output
+        declared = getattr(interface, "region_output_cotangent_constant_over_positions", None)
+        if declared is False:
+            return g_region_output
         first = g_region_output[:, :, :1].expand_as(g_region_output)
-        known = self._constant_over_positions.get(type(interface)) if self.position_constant_update == "verify_once" else None
-        if known is None:
-            known = bool(torch.equal(first, g_region_output))
-            self._constant_over_positions[type(interface)] = known
-        return first if known else g_region_output
+        seq_len = int(g_region_output.shape[2])
+        if self.position_constant_update == "verify_once":
+            try:
+                seen = self._constant_over_positions.setdefault(interface, {})
+            except TypeError:  # an interface object that cannot be weakly referenced: check every time
+                seen = {}
+            if seen.get(seq_len):
+                return first
+            flags = torch.stack([(first == g_region_output).all(), (g_region_output != 0).any()]).cpu().tolist()
+            if flags[0] and flags[1]:
+                seen[seq_len] = True
+            return first if flags[0] else g_region_output
+        return first if bool(torch.equal(first, g_region_output)) else g_region_output
 
     def region_state_jacobian_t(self, *, model: Any, region_cache: Any) -> torch.Tensor:
         state_in = region_cache.state_in
@@ -89,12 +106,109 @@ class StructuredInterfacePullbackProvider:
         return [self.region_state_jacobian_t(model=model, region_cache=rc) for rc in region_caches]
 
 
-def build_interface_pullback_provider(mode: str, *, basis_chunk: int = 0,
-                                      position_constant_update: str = "verify_once") -> StructuredInterfacePullbackProvider:
-    """Name lookup in the style of reference backward/pullbacks.py:185-197; the autograd
-    providers of the reference stay in the reference."""
+class TorchGraphInterfacePullbackProvider:
+    """``Jt`` per region from the forward graph held by ``cache["states"]`` (the reference's default provider,
+    backward/pullbacks.py:37-81, 152-165): ``d`` vector-Jacobian products of ``s_{r+1}`` with respect to
+    ``s_r``, batched through ``is_grads_batched`` where every operator on the way supports it, one at a time
+    otherwise.  Plain ``torch.autograd`` on whatever device the states live on; no kernel of this package is
+    involved until the matrices reach the scan."""
+
+    name = "torch_graph"
+
+    def __init__(self, *, basis_chunk: int = 1) -> None:
+        self.basis_chunk = int(basis_chunk)
+
+    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
+        states = cache["states"]
+        if len(states) != model.num_regions + 1:
+            raise ValueError("cache has invalid states length.")
+        result = []
+        for s_in, s_out in zip(states[:-1], states[1:]):
+            if s_in.dim() != 2 or s_out.dim() != 2:
+                raise ValueError("interface states must be [B, R].")
+            bsz, rank = s_out.shape
+            eye = torch.eye(rank, device=s_out.device, dtype=s_out.dtype)
+
+            def vjp(seed, batched):
+                return torch.autograd.grad(s_out, s_in, grad_outputs=seed, retain_graph=True, create_graph=False,
+                                           allow_unused=False, is_grads_batched=batched)[0]
+
+            try:
+                rows = vjp(eye.unsqueeze(1).expand(rank, bsz, rank), True)        # [j, B, i]
+                result.append(rows.permute(1, 2, 0).contiguous())
+            except (TypeError, RuntimeError) as exc:
+                if isinstance(exc, RuntimeError) and "doesn't have storage" not in str(exc):
+                    raise
+                cols = [vjp(eye[j].expand(bsz, rank), False) for j in range(rank)]
+                result.append(torch.stack(cols, dim=-1))
+        return result
+
+
+class TorchRecomputeInterfacePullbackProvider:
+    """``Jt`` per region by re-running the region on a replicated batch (the reference's ``recompute`` mode,
+    backward/pullbacks.py:84-149, 168-182): ``basis_chunk`` copies of the batch go through decode -> region ->
+    update again, and one backward pass seeded with that many basis vectors yields as many columns.  Needs
+    no forward graph in the cache.  Plain ``torch.autograd``, as above."""
+
+    name = "torch_recompute"
+
+    def __init__(self, *, basis_chunk: int = 1) -> None:
+        self.basis_chunk = int(basis_chunk)
+
+    @staticmethod
+    def _state_map(model: Any, region_index: int, canvas: torch.Tensor, state: torch.Tensor) -> torch.Tensor:
+        condition = model.interface.decode(state, region_index)
+        region_output, _ = model.region_backend.forward_region(region_input=canvas + condition.unsqueeze(1),
+                                                               region_index=region_index)
+        return model.interface.update(state, region_output, region_index).state
+
+    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
+        if self.basis_chunk <= 0:
+            raise ValueError("basis_chunk must be > 0.")
+        region_caches = cache["region_caches"]
+        if len(region_caches) != model.num_regions:
+            raise ValueError("cache has invalid region_caches length.")
+        result = []
+        for rc in region_caches:
+            state, canvas = rc.state_in.detach(), rc.canvas_features.detach()
+            if state.dim() != 2:
+                raise ValueError("interface state inputs must be [B, R].")
+            if canvas.dim() != 3:
+                raise ValueError("canvas_features must be [B, L, D].")
+            bsz, rank = state.shape
+            if canvas.shape[0] != bsz:
+                raise ValueError("canvas_features and state batch sizes do not match.")
+            eye = torch.eye(rank, device=state.device, dtype=state.dtype)
+            cols = []
+            for start in range(0, rank, self.basis_chunk):
+                basis = eye[start:start + self.basis_chunk]
+                n = int(basis.shape[0])
+                with torch.enable_grad():
+                    state_rep = state.repeat(n, 1).requires_grad_(True)               # copy c holds rows c*B..c*B+B-1
+                    out_rep = self._state_map(model, rc.region_index, canvas.repeat(n, 1, 1), state_rep)
+                    seed = basis.repeat_interleave(bsz, dim=0).to(device=out_rep.device, dtype=out_rep.dtype)
+                    (g_in,) = torch.autograd.grad(out_rep, state_rep, grad_outputs=seed)
+                cols.append(g_in.reshape(n, bsz, rank).permute(1, 2, 0))
+            result.append(torch.cat(cols, dim=-1).to(device=state.device, dtype=state.dtype).contiguous())
+        return result
+
+
+def build_interface_pullback_provider(mode: str, *, basis_chunk: int | None = None,
+                                      position_constant_update: str = "verify_once"):
+    """Provider by name.  ``graph`` / ``recompute`` and their aliases are the reference's modes
+    (backward/pullbacks.py:185-197; the values its configuration field ``interface_jacobian_mode`` takes) and
+    give the autograd providers above; ``structured`` (aliases ``hip``, ``structured_hip``) gives the provider
+    that runs the region pullback on the HIP kernels, for which ``basis_chunk`` counts directions per call.
+    ``basis_chunk=None`` means the reference's default of 1 for the autograd providers and 0 (all ``d``
+    directions in one call) for the structured one."""
     normalized = str(mode).strip().lower().replace("-", "_")
     if normalized in {"structured", "hip", "structured_hip"}:
-        return StructuredInterfacePullbackProvider(basis_chunk=basis_chunk,
+        return StructuredInterfacePullbackProvider(basis_chunk=0 if basis_chunk is None else basis_chunk,
                                                    position_constant_update=position_constant_update)
-    raise ValueError("interface pullback provider must be one of: structured, hip")
+    basis_chunk = 1 if basis_chunk is None else basis_chunk
+    if normalized in {"graph", "torch_graph", "pytorch_graph"}:
+        return TorchGraphInterfacePullbackProvider(basis_chunk=basis_chunk)
+    if normalized in {"recompute", "torch_recompute", "pytorch_recompute"}:
+        return TorchRecomputeInterfacePullbackProvider(basis_chunk=basis_chunk)
+    raise ValueError("interface pullback provider must be one of: graph, recompute, torch_graph, torch_recompute, "
+                     "structured, hip")

@@ -1,40 +1,51 @@
-"""Exact scan backward step of an LBI model on the HIP scan kernels.
+"""Exact scan backward step of an LBI model on the HIP scan kernels, and the engine around it.
 
-Counterpart of ``lbi_scan_backward_step`` (reference backward/scan.py:18-97): same
-arguments and result, same order of calls into the local-VJP provider, same edge cases
-(no region: ``RuntimeError``; one region: no Jacobian is built).  What differs is the middle:
+Counterparts of ``lbi_scan_backward_step`` and ``ScanADEngine`` / ``ReferenceScanEngine``
+(reference backward/scan.py:18-97, :100-171): same arguments, defaults, results and diagnostics
+keys, same order of calls into the local-VJP provider, same edge cases (no region:
+``RuntimeError``; one region: no Jacobian is built).  What differs is the middle:
 
-* the state adjoints come from one launch of the cotangent chain (no ``d x d`` product,
-  no list of K+1 suffix matrices); the suffix matrices are formed only when the Jacobian
-  statistics ask for them;
-* the reference recomputes the chain a second time with K sequential mat-vecs on every
-  step to report ``interface_scan_rms`` (:63-72), which costs K launches and a host
-  synchronisation.  Here that cross-check is opt-in (``check_scan=True``): it compares the
-  chain with the adjoints obtained from materialised suffix matrices, the two independent
-  device paths; off, ``interface_scan_rms`` is 0.0.
+* the state adjoints and the suffix matrices come from ONE launch
+  (``lbi_suffix_scan_with_cotangents``): the adjoints are the chain ``g_r = Jt_r g_{r+1}`` carried
+  beside the matrix products;
+* ``interface_scan_rms`` (logged by the reference's training loop as ``scan_align``) is reported
+  on every step as the reference does (:63-72), from the two independent results that launch
+  yields: the chain, and the suffix matrices applied to the last cotangent (one more launch
+  for all regions together, one reduction, one scalar read - where the reference spends K
+  mat-vec launches and the same read).  ``check_scan=False`` skips it (no suffix matrix is formed,
+  no host synchronisation, 0.0 reported) for callers that do not log it.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
 from typing import Any
 
 import torch
+from torch import nn
 
+from ..hip.interface import suffix_scan_cotangents, suffix_scan_pullbacks_and_cotangents
+from .base import ADResult, LBIBackwardResult, ScanBackpropModel, assign_grad_map
+from .local_vjp import TorchAutogradLocalVJPProvider
+from .pullbacks import build_interface_pullback_provider
 from .suffix_scan import (
+    _stack_for_chain,
     interface_state_jacobian_t_stats,
     propagate_state_adjoint_from_last_region_input,
 )
 
-GradMap = dict
 
-
-@dataclass
-class LBIBackwardResult:
-    """Same fields as reference backward/base.py:19-23."""
-
-    grad_map: GradMap
-    interface_scan_rms: float
-    interface_jacobian_stats: dict[str, float] | None = None
+def _adjoints_and_scan_rms(state_jacobians_t, g_last_input: torch.Tensor) -> tuple[list[torch.Tensor], float]:
+    """State adjoints of every region input plus the RMS difference between the two ways of getting them."""
+    stacked = _stack_for_chain(state_jacobians_t[:-1])            # the last region's output state is unused
+    bsz, count, rank, _ = stacked.shape
+    suffix, chain = suffix_scan_pullbacks_and_cotangents(stacked, g_last_input)
+    g32 = g_last_input.to(device=stacked.device, dtype=torch.float32)
+    # suffix[b, r] @ g[b] for all (b, r) at once: B*count one-step chains
+    applied = suffix_scan_cotangents(suffix[:, :count].reshape(bsz * count, 1, rank, rank),
+                                     g32.repeat_interleave(count, dim=0))[:, 0].reshape(bsz, count, rank)
+    # mean over the count + 1 regions of the per-region mean square; the last region's entry is g in both lists
+    rms = torch.sqrt(((applied - chain[:, :count]) ** 2).sum() / float(bsz * (count + 1) * rank))
+    adjoints = [chain[:, r].to(g_last_input.dtype) for r in range(count + 1)]
+    return adjoints, float(rms.item())
 
 
 def lbi_scan_backward_step(
@@ -43,11 +54,13 @@ def lbi_scan_backward_step(
     ce_loss: torch.Tensor,
     cache: dict[str, Any],
     pullback_provider: Any,
-    local_vjp_provider: Any,
+    local_vjp_provider: Any | None = None,
     compute_interface_jacobian_stats: bool = False,
     include_interface_jacobian_suffix: bool = False,
-    check_scan: bool = False,
+    check_scan: bool = True,
 ) -> LBIBackwardResult:
+    """Exact scan backward for an LBI model using a supplied interface-pullback provider."""
+    local_vjp_provider = local_vjp_provider or TorchAutogradLocalVJPProvider()
     grad_map = local_vjp_provider.new_grad_map(model)
     states = list(cache["states"])
     num_regions = len(list(cache["region_ranges"]))
@@ -67,13 +80,13 @@ def lbi_scan_backward_step(
         if compute_interface_jacobian_stats:
             interface_jacobian_stats = interface_state_jacobian_t_stats(
                 state_jacobians_t, include_suffix=include_interface_jacobian_suffix)
-        g_state_inputs = propagate_state_adjoint_from_last_region_input(
-            state_jacobians_t, g_last_input, num_regions=num_regions)
+        if len(state_jacobians_t) != num_regions:
+            raise ValueError("state_jacobians_t length mismatch.")
         if check_scan:
-            g_check = propagate_state_adjoint_from_last_region_input(
-                state_jacobians_t, g_last_input, num_regions=num_regions, materialize_suffix=True)
-            diffs = [((a.float() - b.float()) ** 2).mean() for a, b in zip(g_state_inputs, g_check)]
-            interface_scan_rms = float(torch.sqrt(torch.stack(diffs).mean()).item())
+            g_state_inputs, interface_scan_rms = _adjoints_and_scan_rms(state_jacobians_t, g_last_input)
+        else:
+            g_state_inputs = propagate_state_adjoint_from_last_region_input(
+                state_jacobians_t, g_last_input, num_regions=num_regions)
 
     local_vjp_provider.store_initial_interface_grads(
         model=model, state0=states[0], state0_adjoint=g_state_inputs[0], grad_map=grad_map)
@@ -84,3 +97,71 @@ def lbi_scan_backward_step(
     local_vjp_provider.store_shared_canvas_grads(model=model, loss=ce_loss, grad_map=grad_map)
     return LBIBackwardResult(grad_map=grad_map, interface_scan_rms=interface_scan_rms,
                              interface_jacobian_stats=interface_jacobian_stats)
+
+
+class ScanADEngine:
+    """The engine the reference's training loop builds every step (train/runners.py:368-372): holds the two
+    providers and the diagnostics switches, ``backward`` runs the step and writes ``param.grad``.  Constructor
+    and ``from_config`` take the reference's arguments (backward/scan.py:103-136); ``state_jacobian_mode``
+    also accepts ``"structured"`` for the provider that runs on the HIP region pullback."""
+
+    name = "scan"
+
+    def __init__(
+        self,
+        *,
+        pullback_provider: Any | None = None,
+        local_vjp_provider: Any | None = None,
+        state_jacobian_mode: str = "graph",
+        state_jacobian_basis_chunk: int = 1,
+        compute_interface_jacobian_stats: bool = False,
+        include_interface_jacobian_suffix: bool = False,
+    ) -> None:
+        self.pullback_provider = pullback_provider or build_interface_pullback_provider(
+            state_jacobian_mode, basis_chunk=state_jacobian_basis_chunk)
+        self.local_vjp_provider = local_vjp_provider or TorchAutogradLocalVJPProvider()
+        self.compute_interface_jacobian_stats = bool(compute_interface_jacobian_stats)
+        self.include_interface_jacobian_suffix = bool(include_interface_jacobian_suffix)
+
+    @classmethod
+    def from_config(cls, cfg: Any, *, compute_interface_jacobian_stats: bool = False) -> "ScanADEngine":
+        """Reads ``interface_jacobian_mode``, ``jacobian_basis_chunk`` and ``log_interface_jacobian_suffix``
+        of the reference's training configuration (train/config.py:164-171)."""
+        return cls(
+            pullback_provider=build_interface_pullback_provider(
+                str(cfg.interface_jacobian_mode), basis_chunk=int(cfg.jacobian_basis_chunk)),
+            local_vjp_provider=TorchAutogradLocalVJPProvider(),
+            compute_interface_jacobian_stats=compute_interface_jacobian_stats,
+            include_interface_jacobian_suffix=bool(cfg.log_interface_jacobian_suffix),
+        )
+
+    def backward(self, *, model: nn.Module, loss: torch.Tensor, cache: Any | None = None) -> ADResult:
+        if not isinstance(model, ScanBackpropModel):
+            raise TypeError("ScanADEngine requires a model satisfying ScanBackpropModel")
+        if cache is None:
+            raise ValueError("ScanADEngine requires a forward cache")
+        model.zero_grad(set_to_none=True)
+        result = lbi_scan_backward_step(
+            model,
+            ce_loss=loss,
+            cache=cache,
+            pullback_provider=self.pullback_provider,
+            local_vjp_provider=self.local_vjp_provider,
+            compute_interface_jacobian_stats=self.compute_interface_jacobian_stats,
+            include_interface_jacobian_suffix=self.include_interface_jacobian_suffix,
+        )
+        assign_grad_map(model, result.grad_map)
+        diagnostics: dict[str, Any] = {
+            "interface_scan_rms": result.interface_scan_rms,
+            "interface_pullback_provider": self.pullback_provider.name,
+            "local_vjp_provider": self.local_vjp_provider.name,
+        }
+        if result.interface_jacobian_stats is not None:
+            diagnostics["interface_jacobian_stats"] = dict(result.interface_jacobian_stats)
+        return ADResult(grad_map=result.grad_map, diagnostics=diagnostics)
+
+
+# The reference names the same class by its role as well (backward/scan.py:170-171).
+ReferenceScanEngine = ScanADEngine
+
+__all__ = ["LBIBackwardResult", "ReferenceScanEngine", "ScanADEngine", "lbi_scan_backward_step"]

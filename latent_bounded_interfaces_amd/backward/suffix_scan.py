@@ -40,13 +40,18 @@ def apply_jacobian_t(
 ) -> torch.Tensor:
     """``result[b] = jacobian_t[b] @ cotangent[b]`` (reference backward/suffix_scan.py:24-38).
 
-    Runs as a one-step cotangent chain on the device; accumulation is fp32 and the
-    result is cast to ``out_dtype`` (default: the cotangent's dtype).
+    Runs as a one-step cotangent chain on the device.  The reference multiplies in
+    ``promote_types(jacobian_t.dtype, cotangent.dtype)``; here the kernel reads fp32 / fp16 / bf16
+    matrices as stored, accumulates in fp32 and the result is cast to ``out_dtype`` (default: the
+    cotangent's dtype).  Any other matrix dtype (fp64 included) is accepted and converted to fp32 first,
+    so an fp64 call keeps the reference's result dtype but carries fp32 accuracy.
     """
     if jacobian_t.dim() != 3 or cotangent.dim() != 2:
         raise ValueError("jacobian_t must be [B, d, d] and cotangent [B, d]")
     if out_dtype is None:
         out_dtype = cotangent.dtype
+    if jacobian_t.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        jacobian_t = jacobian_t.to(torch.float32)
     chain = suffix_scan_cotangents(jacobian_t.unsqueeze(1), cotangent.to(device=jacobian_t.device))
     return chain[:, 0].to(device=cotangent.device, dtype=out_dtype)
 
@@ -113,6 +118,24 @@ def propagate_state_adjoint_from_last_region_input(
     return propagate_state_adjoint_with_jacobian_scan(
         state_jacobians_t[:-1], g_last_input_state, materialize_suffix=materialize_suffix
     )
+
+
+def propagate_state_adjoint_by_autograd_chain(
+    *,
+    states: Sequence[torch.Tensor],
+    top_state_adjoint: torch.Tensor,
+) -> list[torch.Tensor]:
+    """Diagnostic of the reference (backward/suffix_scan.py:82-102): the same adjoints walked through an
+    existing autograd graph, one ``torch.autograd.grad`` per region; no kernel of this package is involved."""
+    if len(states) < 2:
+        raise ValueError("at least two interface states are required.")
+    g_states = [torch.zeros_like(states[0]) for _ in states]
+    g_states[-1] = top_state_adjoint
+    for region_index in reversed(range(len(states) - 1)):
+        (g_states[region_index],) = torch.autograd.grad(
+            states[region_index + 1], states[region_index], grad_outputs=g_states[region_index + 1],
+            retain_graph=True, create_graph=False, allow_unused=False)
+    return g_states
 
 
 def interface_state_jacobian_t_stats(

@@ -88,6 +88,10 @@ LOWP_CASES = [
     # the same kernel at lengths that are no multiple of 32 (zero rows in the last tile, keys past the end masked)
     (37, (1, 2, 1, 64), 2), (38, (2, 1, 255, 64), 3), (39, (1, 2, 127, 128), 2), (40, (1, 1, 31, 64), 1),
     (41, (2, 2, 129, 64), 2), (42, (1, 1, 5, 128), 3),
+    # past the single-launch limits with direction counts that leave the four-kernel path a ragged tail: a last
+    # dQ group of fewer than 8 (Dh = 64) or 4 (Dh = 128) directions, an unpaired last direction in dK/dV
+    (43, (1, 2, 320, 64), 5), (44, (1, 1, 320, 64), 9), (45, (1, 2, 192, 128), 3), (46, (1, 1, 320, 128), 5),
+    (47, (1, 1, 384, 64), 11), (48, (2, 1, 192, 128), 7), (49, (1, 1, 512, 64), 3), (50, (1, 1, 256, 128), 9),
 ]
 
 
@@ -191,3 +195,25 @@ def test_long_context_properties(device):
     want = torch.autograd.grad(out, (qr, kr, vr), grad_outputs=g[:, 3].float())
     for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), want):
         assert _max_rel(a[:, 3], b) <= 2e-2, (name, _max_rel(a[:, 3], b))
+
+
+def test_long_context_full_size_slices_match_oracle(device):
+    """The whole long-context call (bf16, B=4, H=16, T=4096, Dh=128, P=16: 64 (b, h) pairs, 1 GiB of cotangents,
+    3 GiB of results) run once; the first and the last (b, h) pair, two directions each, against per-direction
+    SDPA + autograd of that slice in fp32 on the CPU."""
+    from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis
+
+    bsz, heads, seq, hd, basis = 4, 16, 4096, 128, 16
+    gen = torch.Generator(device=device).manual_seed(0)
+    q, k, v = (torch.randn(bsz, heads, seq, hd, device=device, dtype=torch.bfloat16, generator=gen) for _ in range(3))
+    g = torch.randn(bsz, basis, heads, seq, hd, device=device, dtype=torch.bfloat16, generator=gen)
+    scale = 1.0 / math.sqrt(hd)
+    out = attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, causal=True, kernel_mode="hip")
+    torch.cuda.synchronize()
+    for (b, h), dirs in (((0, 0), (0, 7)), ((bsz - 1, heads - 1), (basis - 1, 6)), ((2, 5), (9, 12))):
+        qs, ks, vs = (t[b:b + 1, h:h + 1].float().cpu() for t in (q, k, v))
+        gs = g[b:b + 1, list(dirs), h:h + 1].float().cpu()
+        want = oattn.attention_pullback_sdpa_loop(qs, ks, vs, gs, softmax_scale=scale, causal=True)
+        for name, a, c in zip(("dq", "dk", "dv"), out, want):
+            got = a[b:b + 1, list(dirs), h:h + 1].float().cpu()
+            assert _max_rel(got, c) <= 2e-2, (name, b, h, _max_rel(got, c))

@@ -1,0 +1,105 @@
+"""The autograd providers and gradient-map helpers of the backward package (CPU: they are plain torch.autograd;
+the scan itself is replaced by the oracle's sequential chain, so no kernel is needed)."""
+from __future__ import annotations
+
+import pytest
+import torch
+
+from latent_bounded_interfaces_amd import backward
+from oracle import lbi_model as olbi
+
+
+def _model(**kw):
+    args = dict(vocab_size=37, dim=16, n_heads=2, n_kv_heads=1, layers=3, layers_per_region=1, interface_width=5,
+                hidden=24, d_conv=3, interface_hidden=7, dtype=torch.float64, seed=11)
+    args.update(kw)
+    return olbi.OracleLBIModel(**args).double()
+
+
+def _batch(seed=5, shape=(2, 7)):
+    gen = torch.Generator().manual_seed(seed)
+    return torch.randint(0, 37, shape, generator=gen), torch.randint(0, 37, shape, generator=gen)
+
+
+@pytest.mark.parametrize("mode,chunk", [("graph", 1), ("recompute", 1), ("recompute", 2), ("recompute", 5), ("recompute", 9)])
+def test_autograd_pullback_providers_match_the_oracle_graph_provider(mode, chunk):
+    model = _model()
+    ids, _ = _batch()
+    _, cache = model.forward_with_cache(ids)
+    want = olbi.GraphInterfacePullbackProvider().materialize_state_jacobian_t(model=model, cache=cache)
+    got = backward.build_interface_pullback_provider(mode, basis_chunk=chunk).materialize_state_jacobian_t(
+        model=model, cache=cache)
+    assert len(got) == len(want) == 3
+    for a, b in zip(got, want):
+        assert a.shape == (2, 5, 5)
+        assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)
+
+
+def test_pullback_provider_errors():
+    model = _model()
+    ids, _ = _batch()
+    _, cache = model.forward_with_cache(ids)
+    with pytest.raises(ValueError, match="states length"):
+        backward.TorchGraphInterfacePullbackProvider().materialize_state_jacobian_t(
+            model=model, cache=dict(cache, states=cache["states"][:-1]))
+    with pytest.raises(ValueError, match="basis_chunk must be > 0"):
+        backward.TorchRecomputeInterfacePullbackProvider(basis_chunk=0).materialize_state_jacobian_t(model=model, cache=cache)
+    with pytest.raises(ValueError, match="region_caches length"):
+        backward.TorchRecomputeInterfacePullbackProvider().materialize_state_jacobian_t(
+            model=model, cache=dict(cache, region_caches=[]))
+
+
+@pytest.mark.parametrize("layers,per_region", [(3, 1), (4, 2), (2, 2)])
+def test_default_local_vjp_provider_reproduces_dense_gradients(layers, per_region):
+    """The reference's parity criterion (tests/test_lbi_gradient_parity.py): scan-step gradients == loss.backward()."""
+    model = _model(layers=layers, layers_per_region=per_region)
+    ids, targets = _batch()
+    _, dense = olbi.dense_gradients(model, ids, targets)
+    logits, cache = model.forward_with_cache(ids)
+    grads = olbi.scan_backward_step_sequential(
+        model, loss=olbi.token_loss(logits, targets), cache=cache,
+        pullback_provider=backward.TorchGraphInterfacePullbackProvider(),
+        local_vjp_provider=backward.TorchAutogradLocalVJPProvider())
+    assert set(grads) == set(dense)
+    for name, want in dense.items():
+        if want is None:
+            assert grads[name] is None
+        else:
+            assert torch.allclose(grads[name], want.to(grads[name].dtype), atol=1e-6, rtol=1e-4), (name, float((grads[name] - want).abs().max()))
+
+
+def test_autograd_chain_diagnostic_matches_the_jacobian_chain():
+    model = _model()
+    ids, targets = _batch()
+    logits, cache = model.forward_with_cache(ids)
+    states = cache["states"]
+    top = torch.randn(2, 5, dtype=torch.float64, generator=torch.Generator().manual_seed(1))
+    got = backward.propagate_state_adjoint_by_autograd_chain(states=states, top_state_adjoint=top)
+    jts = olbi.GraphInterfacePullbackProvider().materialize_state_jacobian_t(model=model, cache=cache)
+    want = top
+    assert torch.equal(got[-1], top)
+    for r in reversed(range(3)):
+        want = torch.einsum("bij,bj->bi", jts[r], want)
+        assert torch.allclose(got[r], want, atol=1e-12)
+    with pytest.raises(ValueError, match="at least two"):
+        backward.propagate_state_adjoint_by_autograd_chain(states=states[:1], top_state_adjoint=top)
+
+
+def test_grad_map_helpers_round_trip():
+    lin = torch.nn.Linear(3, 2)
+    lin.bias.requires_grad_(False)
+    assert backward.collect_named_grads(lin) == {"weight": None}
+    lin(torch.ones(1, 3)).sum().backward()
+    grads = backward.collect_named_grads(lin)
+    assert set(grads) == {"weight"} and torch.equal(grads["weight"], torch.ones(2, 3))
+    grads["weight"] = grads["weight"] * 2
+    backward.assign_grad_map(lin, grads)
+    assert torch.equal(lin.weight.grad, 2 * torch.ones(2, 3)) and lin.weight.grad is not grads["weight"]
+    backward.assign_grad_map(lin, {})
+    assert lin.weight.grad is None
+    target: dict = {}
+    backward.store_named_grads(target, {id(lin.weight): "w"}, [lin.weight], (None,))
+    assert target == {"w": None}
+    result = backward.ADResult(grad_map={})
+    assert result.diagnostics == {}
+    assert backward.LBIBackwardResult(grad_map={}, interface_scan_rms=0.5).interface_jacobian_stats is None

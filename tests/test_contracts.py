@@ -31,6 +31,29 @@ def test_offered_classes_satisfy_their_protocols():
     assert not isinstance(object(), contracts.TransformerLowering)
 
 
+def test_default_providers_and_engine_satisfy_the_protocols():
+    from latent_bounded_interfaces_amd import backward
+
+    assert isinstance(backward.TorchAutogradLocalVJPProvider(), contracts.LocalVJPProvider)
+    for mode, name in (("graph", "torch_graph"), ("recompute", "torch_recompute")):
+        provider = build_interface_pullback_provider(mode)
+        assert isinstance(provider, contracts.InterfacePullbackProvider) and provider.name == name
+        assert provider.basis_chunk == 1
+    engine = backward.ScanADEngine(state_jacobian_mode="recompute", state_jacobian_basis_chunk=32)
+    assert engine.name == "scan" and engine.pullback_provider.basis_chunk == 32
+    assert engine.local_vjp_provider.name == "torch_autograd"
+    assert callable(backward.lbi_reference_scan_backward_step)
+    # every public name of the reference's backward package that lies on this path is importable from here
+    for name in ("ADEngine", "ADResult", "GradMap", "LBIBackwardResult", "ReferenceScanEngine", "ScanADEngine",
+                 "ScanBackpropModel", "TorchAutogradLocalVJPProvider", "TorchGraphInterfacePullbackProvider",
+                 "TorchRecomputeInterfacePullbackProvider", "assign_grad_map", "apply_jacobian_t",
+                 "build_interface_pullback_provider", "collect_named_grads", "compose_suffix_jacobian_t",
+                 "lbi_reference_scan_backward_step", "lbi_scan_backward_step",
+                 "propagate_state_adjoint_by_autograd_chain", "propagate_state_adjoint_from_last_region_input",
+                 "propagate_state_adjoint_with_jacobian_scan", "store_named_grads"):
+        assert hasattr(backward, name), name
+
+
 def test_test_side_providers_satisfy_the_needed_protocols():
     assert isinstance(lbi_model.AutogradLocalVJPProvider(), contracts.LocalVJPProvider)
     assert isinstance(lbi_model.GraphInterfacePullbackProvider(), contracts.InterfacePullbackProvider)

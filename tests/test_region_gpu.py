@@ -461,3 +461,42 @@ def test_kernels_at_the_end_to_end_scale(device):
     assert torch.equal(full[-1, -1], part[0, 0])
     two = region.causal_conv1d_pullback(region.attn_qkv_pullback(dq, dk, dv, **kw), w)
     assert int((two != full).sum()) <= full.numel() // 2000
+
+
+def test_region_pullback_at_the_end_to_end_layer_shape_matches_oracle(device):
+    """Two layers of the end-to-end configuration (d_model 768, 12 heads x 64, hidden 3072, conv 4, T=1024, bf16
+    weights and activations, fp32 residual stream) with B=1 and P=4 against fp32 autograd of the CPU restatement
+    on the same rounded weights: the values behind the full-size timings, not only their indexing."""
+    import copy
+
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+
+    dim, heads, hd, hidden, layers, b, p, t = 768, 12, 64, 3072, 2, 1, 4, 1024
+    dtype = torch.bfloat16
+    backend = oreg.make_backend(dim=dim, n_heads=heads, n_kv_heads=heads, head_dim=hd, hidden=hidden, layers=layers,
+                                d_conv=4, residual_in_fp32=True, dtype=dtype, seed=21)
+    torch.manual_seed(22)
+    x = torch.randn(b, t, dim).to(dtype)
+    basis = torch.randn(b, p, t, dim)
+    ref_backend = copy.deepcopy(backend).float()
+    _, ref_cache = ref_backend.forward_region(region_input=x.float(), region_index=0)
+    want = oreg.input_pullback_basis_autograd(ref_backend, ref_cache, basis)
+    gpu_backend = backend.to(device)
+    with torch.no_grad():
+        _, cache = gpu_backend.forward_region(region_input=x.to(device), region_index=0)
+    low = HipTransformerLowering()
+    got = low.input_pullback_basis(backend=gpu_backend, cache=cache, output_cotangent_basis=basis.to(device))
+    assert _max_rel(got.cpu(), want) <= 2e-2, _max_rel(got.cpu(), want)
+    # the position-constant form a mean-pooling interface produces (stride-0 view over positions)
+    const = torch.randn(b, p, 1, dim)
+    want_c = oreg.input_pullback_basis_autograd(ref_backend, ref_cache, const.expand(b, p, t, dim).contiguous())
+    got_c = low.input_pullback_basis(backend=gpu_backend, cache=cache,
+                                     output_cotangent_basis=const.to(device).expand(b, p, t, dim))
+    assert _max_rel(got_c.cpu(), want_c) <= 2e-2, _max_rel(got_c.cpu(), want_c)
+    # parameter gradients of the same two layers
+    cot = torch.randn(b, t, dim)
+    want_p = oreg.parameter_vjp_autograd(ref_backend, ref_cache, cot)
+    got_p = low.parameter_vjp(backend=gpu_backend, cache=cache, output_cotangent=cot.to(device))
+    assert set(got_p) == set(want_p)
+    for name, w in want_p.items():
+        assert _max_rel(got_p[name].cpu(), w) <= 3e-2, (name, _max_rel(got_p[name].cpu(), w))
