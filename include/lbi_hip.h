@@ -122,6 +122,26 @@ int lbi_attn_pullback(const void* q, const void* k, const void* v, const void* d
                       float softmax_scale, int causal, int dtype, void* stream);
 
 /*
+ * lbi_attn_pullback without a workspace argument and without any allocation: the scratch memory (softmax
+ * statistics, -delta, the fp32 forward output) lives in a static device array of
+ * LBI_ATTN_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.
+ *
+ * This entry has no counterpart in the reference.  It is for callers that cannot allocate device memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Arguments and results
+ * are those of lbi_attn_pullback (the same kernels run, results are bit-identical).  A call whose
+ * lbi_attn_pullback_workspace_bytes(...) exceeds LBI_ATTN_STATIC_SCRATCH_BYTES returns LBI_ERR_WORKSPACE.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
+ * threads) race on it; serialise them.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress), later calls make no runtime call besides the launches.
+ */
+#define LBI_ATTN_STATIC_SCRATCH_BYTES (32u << 20)
+
+int lbi_attn_pullback_static(const void* q, const void* k, const void* v, const void* d_out,
+                             void* dq, void* dk, void* dv,
+                             int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P,
+                             float softmax_scale, int causal, int dtype, void* stream);
+
+/*
  * Region-level input pullback of a Transformer block (the pieces around the matrix products,
  * which the caller issues as plain GEMMs, and around lbi_attn_pullback).  Together they
  * implement TransformerLowering.input_pullback_basis of the reference

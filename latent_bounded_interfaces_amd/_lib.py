@@ -14,7 +14,8 @@ import torch
 LIB_PATH = Path(__file__).resolve().parent / "liblbi_hip.so"
 
 LBI_F32, LBI_F16, LBI_BF16 = 0, 1, 2
-ABI_VERSION = 6
+ATTN_STATIC_SCRATCH_BYTES = 32 << 20  # LBI_ATTN_STATIC_SCRATCH_BYTES of include/lbi_hip.h
+ABI_VERSION = 7
 
 _DTYPE_CODES = {torch.float32: LBI_F32, torch.float16: LBI_F16, torch.bfloat16: LBI_BF16}
 
@@ -44,6 +45,10 @@ SYMBOLS = {
         _c.c_int,
         [_c.c_void_p] * 7 + [_c.c_void_p, _c.c_size_t] + [_c.c_int64] * 5
         + [_c.c_float, _c.c_int, _c.c_int, _c.c_void_p],
+    ),
+    "lbi_attn_pullback_static": (
+        _c.c_int,
+        [_c.c_void_p] * 7 + [_c.c_int64] * 5 + [_c.c_float, _c.c_int, _c.c_int, _c.c_void_p],
     ),
     "lbi_rmsnorm_pullback": (
         _c.c_int,

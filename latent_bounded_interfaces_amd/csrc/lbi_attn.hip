@@ -8,9 +8,36 @@
 #include "lbi_attn_small.h"
 
 #include <cstdlib>
+#include <mutex>
 
 namespace lbi {
 namespace {
+
+// Scratch memory of lbi_attn_pullback_static: one copy per GPU the library runs on, held until the process ends.
+// In host code this name only stands for the symbol; the device address comes from hipGetSymbolAddress, once per
+// device, and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[LBI_ATTN_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** out) {
+    int device = -1;
+    LBI_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices)
+        return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_pullback_static: device index %d out of range", device);
+    std::lock_guard<std::mutex> guard(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void* ptr = nullptr;
+        LBI_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(LBI_ERR_HIP, "lbi_attn_pullback_static: scratch symbol has no device address");
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return LBI_OK;
+}
 
 int check_attn_dims(int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P, int dtype) {
     if (B < 0 || H < 0 || T < 0 || Dh < 0 || P < 0)
@@ -87,4 +114,28 @@ extern "C" int lbi_attn_pullback(const void* q, const void* k, const void* v, co
         case LBI_F16: return attn_generic::launch<_Float16>(q, k, v, d_out, dq, dk, dv, ws, b, h, t, dh, p, softmax_scale, causal, stream);
         default: return attn_generic::launch<bf16_raw>(q, k, v, d_out, dq, dk, dv, ws, b, h, t, dh, p, softmax_scale, causal, stream);
     }
+}
+
+extern "C" int lbi_attn_pullback_static(const void* q, const void* k, const void* v, const void* d_out, void* dq,
+                                        void* dk, void* dv, int64_t B, int64_t H, int64_t T, int64_t Dh, int64_t P,
+                                        float softmax_scale, int causal, int dtype, void* stream_v) {
+    using namespace lbi;
+    clear_error();
+    if (int rc = check_attn_dims(B, H, T, Dh, P, dtype)) return rc;
+    if (B == 0 || H == 0 || T == 0 || Dh == 0 || P == 0) return LBI_OK;
+    if (!q || !k || !v || !d_out || !dq || !dk || !dv)
+        return fail(LBI_ERR_INVALID, "lbi_attn_pullback_static: null tensor pointer");
+    const size_t need = lbi_attn_pullback_workspace_bytes(B, H, T, Dh, P, dtype);
+    if (need > (size_t)LBI_ATTN_STATIC_SCRATCH_BYTES)
+        return fail(LBI_ERR_WORKSPACE,
+                    "lbi_attn_pullback_static: this call needs %zu bytes of scratch memory, the static buffer holds %zu; "
+                    "use lbi_attn_pullback with a caller-provided workspace",
+                    need, (size_t)LBI_ATTN_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (need > 0)
+        if (int rc = static_scratch(&ws)) return rc;
+    // Every kernel of the pullback writes its part of the workspace before any kernel reads it, so what the last
+    // call left behind needs no clearing.
+    return lbi_attn_pullback(q, k, v, d_out, dq, dk, dv, ws, need, B, H, T, Dh, P, softmax_scale, causal, dtype,
+                             stream_v);
 }

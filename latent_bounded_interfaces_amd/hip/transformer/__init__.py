@@ -126,4 +126,40 @@ def attention_input_pullback_basis(
     return dq, dk, dv
 
 
-__all__ = ["attention_input_pullback_basis"]
+def attention_input_pullback_basis_static(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    output_cotangent_basis: torch.Tensor,
+    out: tuple[torch.Tensor, torch.Tensor, torch.Tensor],
+    *,
+    softmax_scale: float,
+    causal: bool = True,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The same pullback written into caller-provided ``out = (dq, dk, dv)`` with no allocation at all (no
+    workspace, no padding, no copies): ``lbi_attn_pullback_static``, whose scratch memory is a static device
+    array of ``_lib.ATTN_STATIC_SCRATCH_BYTES`` per GPU.  For callers that cannot allocate (graph capture, serving
+    loops).  Every tensor must already be contiguous, on one device and of one dtype; a call whose scratch need
+    exceeds the static array raises.  Calls on one GPU share the array and must not overlap in time."""
+    _validate(q, k, v, output_cotangent_basis)
+    tensors = (q, k, v, output_cotangent_basis, *out)
+    if len(out) != 3 or any(o.shape != output_cotangent_basis.shape for o in out):
+        raise ValueError("out must be three tensors shaped like output_cotangent_basis")
+    if not all(t.is_cuda and t.device == q.device and t.dtype == q.dtype and t.is_contiguous() for t in tensors):
+        raise RuntimeError("all tensors must be contiguous CUDA tensors of one dtype on one device")
+    if output_cotangent_basis.numel() == 0:
+        return out
+    bsz, heads, seqlen, head_dim = q.shape
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        status = lib.lbi_attn_pullback_static(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), output_cotangent_basis.data_ptr(),
+            out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr(),
+            bsz, heads, seqlen, head_dim, output_cotangent_basis.shape[1],
+            float(softmax_scale), int(bool(causal)), _lib.dtype_code(q.dtype), _lib.current_stream_ptr(q.device),
+        )
+    _lib.check(status, "lbi_attn_pullback_static")
+    return out
+
+
+__all__ = ["attention_input_pullback_basis", "attention_input_pullback_basis_static"]

@@ -96,6 +96,15 @@ def test_region_and_norm_entry_points_validate_on_the_host():
     assert lib.lbi_attn_pullback_workspace_bytes(8, 8, 128, 64, 4, f32) > 0
     assert lib.lbi_attn_pullback(one, one, one, one, one, one, one, None, 0, 8, 8, 320, 64, 4, 0.125, 1, f16, None) == -4
     assert b"workspace" in lib.lbi_last_error()
+    # the allocation-free entry rejects, on the host, what its static scratch array cannot hold
+    assert lib.lbi_attn_pullback_workspace_bytes(4, 16, 4096, 128, 16, _lib.LBI_BF16) > _lib.ATTN_STATIC_SCRATCH_BYTES
+    assert lib.lbi_attn_pullback_static(one, one, one, one, one, one, one, 4, 16, 4096, 128, 16, 0.1, 1,
+                                        _lib.LBI_BF16, None) == -4
+    assert b"static buffer holds" in lib.lbi_last_error()
+    assert lib.lbi_attn_pullback_static(None, one, one, one, one, one, one, 1, 1, 320, 64, 1, 0.1, 1, f16, None) == -1
+    assert lib.lbi_attn_pullback_static(None, None, None, None, None, None, None, 0, 1, 320, 64, 1, 0.1, 1, f16, None) == 0
+    header = HEADER.read_text()
+    assert f"#define LBI_ATTN_STATIC_SCRATCH_BYTES ({_lib.ATTN_STATIC_SCRATCH_BYTES >> 20}u << 20)" in header
 
 
 def test_wrappers_reject_bad_input_before_touching_the_device():
