@@ -405,16 +405,16 @@ template <int DH> constexpr size_t dkdv_pair_lds_bytes() {
 }
 
 template <typename T, int DH, bool CAUSAL>
-void launch_dkdv_pair(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk,
+int launch_dkdv_pair(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk,
                       T* dv, int n_bh, int H, int P, int T_len, float scale, hipStream_t stream) {
     const int n_kb = (T_len + 127) / 128;
     const int n_pp = (P + 1) / 2;
     constexpr size_t lds_bytes = dkdv_pair_lds_bytes<DH>();
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dkdv_pair_kernel<T, DH, CAUSAL>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (int rc = ensure_dynamic_lds<&dkdv_pair_kernel<T, DH, CAUSAL>>(lds_bytes)) return rc;
     hipLaunchKernelGGL((dkdv_pair_kernel<T, DH, CAUSAL>), dim3(grid_size(n_kb * n_pp, n_bh)), dim3(256), lds_bytes,
                        stream, q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale);
+    return LBI_OK;
 }
 
 }  // namespace attn_mfma

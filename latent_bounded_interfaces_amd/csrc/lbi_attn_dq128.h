@@ -252,17 +252,17 @@ template <int DH, int PB> constexpr size_t dq_ring_lds_bytes() {
 // PB is the direction block of the caller's choice (1, 2, 4, and 8 for head dim 64); head dim 128 has
 // accumulation registers for four.
 template <typename T, int DH, int PB, bool CAUSAL>
-void launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
+int launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
                int H, int P, int T_len, float scale, hipStream_t stream) {
     constexpr int PBK = (DH == 128 && PB > 4) ? 4 : PB;
     const int n_qb = (T_len + 127) / 128;
     const int n_pb = (P + PBK - 1) / PBK;
     constexpr size_t lds_bytes = dq_ring_lds_bytes<DH, PBK>();
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(dq_ring_kernel<T, DH, PBK, CAUSAL>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (int rc = ensure_dynamic_lds<&dq_ring_kernel<T, DH, PBK, CAUSAL>>(lds_bytes)) return rc;
     hipLaunchKernelGGL((dq_ring_kernel<T, DH, PBK, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), lds_bytes,
                        stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
+    return LBI_OK;
 }
 
 }  // namespace attn_mfma

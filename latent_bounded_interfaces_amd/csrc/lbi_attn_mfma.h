@@ -367,17 +367,17 @@ inline size_t workspace_floats(int64_t B, int64_t H, int64_t T, int64_t Dh, int6
 
 // dK/dV launch (kernel in lbi_attn_dkdv128.h).
 template <typename T, int DH, bool CAUSAL>
-void launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
+int launch_dkdv(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk, T* dv,
                  int n_bh, int H, int P, int T_len, float scale, hipStream_t stream);
 
 // dK/dV launch for two or more directions (kernel in lbi_attn_dkdv_pair.h).
 template <typename T, int DH, bool CAUSAL>
-void launch_dkdv_pair(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk,
+int launch_dkdv_pair(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dk,
                       T* dv, int n_bh, int H, int P, int T_len, float scale, hipStream_t stream);
 
 // dQ launch (kernel in lbi_attn_dq128.h); PB = directions per wave.
 template <typename T, int DH, int PB, bool CAUSAL>
-void launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
+int launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
                int H, int P, int T_len, float scale, hipStream_t stream);
 
 template <typename T, int DH, bool CAUSAL>
@@ -395,12 +395,15 @@ int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T
     hipLaunchKernelGGL((delta_kernel<T, DH>), dim3((unsigned)((T_len + rows_per_block - 1) / rows_per_block) * n_bh),
                        dim3(256), 0, stream, g, o32, delta, H, P, T_len);
     // directions per wave of the dQ kernel: as many as share one S tile, without idle slots for one or two directions
-    if (P == 1) launch_dq<T, DH, 1, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    else if (P == 2) launch_dq<T, DH, 2, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    else if (DH == 64 && P > 4) launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    else launch_dq<T, DH, 4, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    if (P >= 2) launch_dkdv_pair<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
-    else launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
+    int rc;
+    if (P == 1) rc = launch_dq<T, DH, 1, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else if (P == 2) rc = launch_dq<T, DH, 2, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else if (DH == 64 && P > 4) rc = launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else rc = launch_dq<T, DH, 4, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    if (rc) return rc;
+    if (P >= 2) rc = launch_dkdv_pair<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
+    else rc = launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
+    if (rc) return rc;
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }

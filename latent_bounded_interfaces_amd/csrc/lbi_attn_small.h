@@ -261,14 +261,17 @@ int launch_sized(const void* q, const void* k, const void* v, const void* g, voi
     const int n_bh = B * H;
     const dim3 grid(grid_size(P, n_bh));
     auto run = [&](auto kern) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)lds);
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, static_cast<const T*>(q), static_cast<const T*>(k),
                            static_cast<const T*>(v), static_cast<const T*>(g), static_cast<T*>(dq), static_cast<T*>(dk),
                            static_cast<T*>(dv), n_bh, H, P, T_len, scale);
     };
-    if (causal) run(small_seq_kernel<T, DH, MAX_TILES, true>);
-    else run(small_seq_kernel<T, DH, MAX_TILES, false>);
+    if (causal) {
+        if (int rc = ensure_dynamic_lds<&small_seq_kernel<T, DH, MAX_TILES, true>>(lds)) return rc;
+        run(small_seq_kernel<T, DH, MAX_TILES, true>);
+    } else {
+        if (int rc = ensure_dynamic_lds<&small_seq_kernel<T, DH, MAX_TILES, false>>(lds)) return rc;
+        run(small_seq_kernel<T, DH, MAX_TILES, false>);
+    }
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/lbi_hip.h"
 
 namespace lbi {
@@ -23,6 +25,25 @@ inline size_t dtype_size(int dtype) {
         if (lbi_e_ != hipSuccess)                                                        \
             return ::lbi::fail(LBI_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(lbi_e_)); \
     } while (0)
+
+// Raises the dynamic-LDS limit of kernel KERN to `bytes` where the default 64 KiB does not do.  The runtime call is
+// made once per kernel and device (a later, larger request raises it again); launches after that only read a flag,
+// so nothing but the launch itself happens on a hot path or inside a stream capture.  A failure is reported, not
+// left for the launch to trip over.
+template <auto KERN>
+int ensure_dynamic_lds(size_t bytes) {
+    constexpr int kTracked = 32;
+    static std::atomic<size_t> granted[kTracked];  // zero-initialised
+    if (bytes <= 64 * 1024) return LBI_OK;
+    int dev = 0;
+    LBI_HIP_CHECK(hipGetDevice(&dev));
+    const bool tracked = dev >= 0 && dev < kTracked;
+    if (tracked && granted[dev].load(std::memory_order_relaxed) >= bytes) return LBI_OK;
+    LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(KERN), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)bytes));
+    if (tracked) granted[dev].store(bytes, std::memory_order_relaxed);
+    return LBI_OK;
+}
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));

@@ -46,10 +46,31 @@ namespace {
 // fragments of mats[r] that feed the MFMAs are already in registers, so a step costs
 // D/2 extra FMAs per lane (and nothing from HBM); every column block computes the chain,
 // block 0 writes it.
-template <typename Tin, int D, int RT, int CB, bool COT>
+// Which part of the chain a workgroup runs.  `phase` 0 is the whole chain of a batch element (K - 1 dependent
+// steps).  Phases 1-3 are the K-parallel form for batches too small to fill the chip with one chain per column
+// block: the chain is cut into C chunks of L matrices and
+//   phase 1  every chunk c >= 1 multiplies its own matrices (L - 1 steps, all chunks side by side): the last chunk's
+//            products are final results and are stored as in phase 0; a middle chunk keeps only its total
+//            T_c = mats[cL] ... mats[(c+1)L - 1], parked in out[cL + 1], a slot phase 3 rewrites;
+//   phase 2  one chain over the totals (C - 2 steps): out[cL] = T_c @ out[(c+1)L] for c = C-2 ... 1, which are the
+//            final suffix products at the chunk boundaries (the kernel runs it with mats = the parked totals);
+//   phase 3  every chunk c <= C-2 restarts the chain from out[(c+1)L] through its own matrices (L - 1 or, for chunk
+//            0, L steps, all chunks side by side), storing each product.
+// The cotangents, if asked for, are then the finished products applied to g (suffix_apply_kernel).
+// About twice the products, a dependent depth of 2L + C - 3 instead of K - 1, no scratch memory, no atomics; the
+// summation order is fixed by (K, L), so reruns are bit-identical.
+struct ScanPlan {
+    int phase;  // 0: whole chain; 1, 2, 3: see above
+    int L;      // matrices per chunk (>= 2)
+    int C;      // chunks (>= 3)
+};
+
+// MODE 0: phase 0 only; every switch below is a compile-time constant, which keeps the whole-chain kernel at its
+// register count.  MODE 1: phases 1 and 3 (switches at run time, unit strides).  MODE 2: phase 2 (strided).
+template <typename Tin, int D, int RT, int CB, bool COT, int MODE>
 __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     const Tin* __restrict__ mats, float* __restrict__ out, const float* __restrict__ g,
-    float* __restrict__ cot, int B, int K) {
+    float* __restrict__ cot, int B, int K, ScanPlan plan) {
     constexpr int NW = D / RT;          // waves per workgroup
     constexpr int NT = 64 * NW;         // threads
     constexpr int RTILES = RT / 32;
@@ -57,17 +78,29 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     constexpr int NB = D / CB;          // column blocks per batch element
     constexpr int PITCH = D + 4;
     constexpr int NCH = D / 32;         // k chunks per step
+    constexpr size_t DD = (size_t)D * D;
 
     extern __shared__ __align__(16) float lds[];  // [2][CB][PITCH], then (COT) [2][D]
     float* vbuf = lds + 2 * CB * PITCH;
 
-    // Workgroups are dealt round-robin to the 8 XCDs; all column blocks of one
-    // batch element get ids that are equal mod 8 so they share one L2.
+    // A launch covers E = B * (segments per batch element) chains.  With at least 8 of them the workgroups are
+    // dealt round-robin to the 8 XCDs so that all column blocks of one chain get ids that are equal mod 8 and
+    // share one L2; smaller launches are sized exactly.
+    const int nseg = MODE == 1 ? plan.C - 1 : 1;
+    const int E = B * nseg;
     const int id = blockIdx.x;
-    const int slot = id >> 3;
-    const int b = (slot / NB) * 8 + (id & 7);
-    const int c0 = (slot % NB) * CB;
-    if (b >= B) return;
+    int e, c0;
+    if (E >= 8) {
+        const int slot = id >> 3;
+        e = (slot / NB) * 8 + (id & 7);
+        c0 = (slot % NB) * CB;
+    } else {
+        e = id / NB;
+        c0 = (id % NB) * CB;
+    }
+    if (e >= E) return;
+    const int b = e / nseg;
+    const int seg = e - b * nseg;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -76,30 +109,78 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     const int h = lane >> 5;
     const int row0 = wave * RT;
 
-    const Tin* mats_b = mats + (size_t)b * K * D * D;
-    float* out_b = out + (size_t)b * (K + 1) * D * D;
+    float* out_b = out + (size_t)b * (K + 1) * DD;
+    // The chain of this workgroup: steps r = r_top ... r_lo multiply a_base[r * a_stride] onto the running suffix
+    // and store it at o_base[r * o_stride]; the suffix starts as the matrix `init_a` (storage type) or `init_s`
+    // (fp32, a product computed earlier).
+    const Tin* a_base = mats + (size_t)b * K * DD;
+    float* o_base = out_b;
+    const Tin* init_a = nullptr;
+    const float* init_s = nullptr;
+    int r_top, r_lo = 0;
+    bool write_tail = false;   // the start matrix and the identity behind it are results (out[K - 1], out[K])
+    bool store_all = true;     // every step's product is a result
+    bool cot_on = COT;         // the cotangent chain of this workgroup is a result
+    bool cot_init = false;     // ... including its first vector (init_s @ g)
+    size_t stride_rt = DD;
+    if constexpr (MODE == 0) {
+        init_a = a_base + (size_t)(K - 1) * DD;
+        r_top = K - 2;
+        write_tail = true;
+    } else if constexpr (MODE == 1) {
+        if (plan.phase == 1) {
+            const int c = seg + 1;
+            const bool last = c == plan.C - 1;
+            const int end = last ? K : (c + 1) * plan.L;
+            init_a = a_base + (size_t)(end - 1) * DD;
+            r_top = end - 2;
+            r_lo = c * plan.L;
+            write_tail = last;
+            store_all = last;
+            cot_on = COT && last;
+        } else {
+            const int c = seg;
+            init_s = out_b + (size_t)(c + 1) * plan.L * DD;
+            r_top = (c + 1) * plan.L - 1;
+            r_lo = c == 0 ? 0 : c * plan.L + 1;   // out[cL] is a phase 2 result already
+            cot_init = c < plan.C - 2;            // out[(C-1)L] @ g is the last chunk's own chain value
+        }
+    } else {
+        // step j multiplies the total parked in out[(j+1)L + 1] and stores out[(j+1)L]
+        a_base = reinterpret_cast<const Tin*>(out_b + (size_t)(plan.L + 1) * DD);
+        o_base = out_b + (size_t)plan.L * DD;
+        stride_rt = (size_t)plan.L * DD;
+        init_s = out_b + (size_t)(plan.C - 1) * plan.L * DD;
+        r_top = plan.C - 3;
+        cot_on = false;
+    }
+    const bool from_a = MODE == 0 || (MODE == 1 && plan.phase == 1);  // start state: init_a, else init_s
+    // distance between the matrices (and the results) of consecutive steps: a constant except in phase 2
+    const size_t a_stride = MODE == 2 ? stride_rt : DD;
+    const size_t o_stride = a_stride;
 
-    // Identity tail and the first suffix (= mats[K-1]); fill St buffer 0.
+    // Start state into St buffer 0 (and, with write_tail, to its place in the result with the identity behind it).
     {
-        const Tin* a_last = mats_b + (size_t)(K - 1) * D * D;
-        float* o_last = out_b + (size_t)(K - 1) * D * D;
-        float* o_eye = out_b + (size_t)K * D * D;
+        float* o_last = out_b + (size_t)(K - 1) * DD;
+        float* o_eye = out_b + (size_t)K * DD;
         for (int idx = tid; idx < D * CB; idx += NT) {
             const int row = idx / CB;
             const int col = idx % CB;
-            const float val = to_f32(a_last[row * D + c0 + col]);
-            o_last[row * D + c0 + col] = val;
-            o_eye[row * D + c0 + col] = (row == c0 + col) ? 1.0f : 0.0f;
+            const float val = from_a ? to_f32(init_a[row * D + c0 + col]) : init_s[row * D + c0 + col];
+            if (write_tail) {
+                o_last[row * D + c0 + col] = val;
+                o_eye[row * D + c0 + col] = (row == c0 + col) ? 1.0f : 0.0f;
+            }
             lds[col * PITCH + row] = val;
         }
         if (COT) {
-            // v[K] = g and v[K-1] = mats[K-1] @ g (one row per thread, once per kernel)
+            // first vector of the chain: (start state) @ g, one row per thread, once per kernel
             const float* g_b = g + (size_t)b * D;
             float* cot_b = cot + (size_t)b * (K + 1) * D;
             for (int row = tid; row < D; row += NT) {
                 float acc = 0.0f;
                 for (int k4 = 0; k4 < D; k4 += 4) {
-                    const f32x4 a4 = load4(a_last + row * D + k4);
+                    const f32x4 a4 = from_a ? load4(init_a + row * D + k4) : load4(init_s + row * D + k4);
                     acc = fmaf(a4[0], g_b[k4], acc);
                     acc = fmaf(a4[1], g_b[k4 + 1], acc);
                     acc = fmaf(a4[2], g_b[k4 + 2], acc);
@@ -107,14 +188,17 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 }
                 vbuf[row] = acc;
                 if (c0 == 0) {
-                    cot_b[(size_t)K * D + row] = g_b[row];
-                    cot_b[(size_t)(K - 1) * D + row] = acc;
+                    if (write_tail && cot_on) {
+                        cot_b[(size_t)K * D + row] = g_b[row];
+                        cot_b[(size_t)(K - 1) * D + row] = acc;
+                    }
+                    if (cot_init) cot_b[(size_t)(r_top + 1) * D + row] = acc;
                 }
             }
         }
     }
     __syncthreads();
-    if (K < 2) return;
+    if (r_top < r_lo) return;
 
     // Lane's slice of mats[r]: rows row0 + 32*i + m, k = 32*kc + 16*h + [0, 16).
     auto load_a = [&](f32x4 (&dst)[RTILES][4], const Tin* base) {
@@ -123,28 +207,28 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
 #pragma unroll
             for (int q = 0; q < 4; ++q) dst[i][q] = load4(base + (size_t)i * 32 * D + q * 4);
     };
-    const Tin* a_lane = mats_b + (size_t)(row0 + m) * D + h * 16;  // + r*D*D + kc*32
+    const Tin* a_lane = a_base + (size_t)(row0 + m) * D + h * 16;  // + r*a_stride + kc*32
 
     // mats chunks are prefetched RING-1 chunks ahead into a register ring; the ring
     // index of a chunk is kc % RING, the same in every step because RING divides NCH.
     constexpr int RING = (NCH % 4 == 0) ? 4 : 2;
     constexpr int AHEAD = RING - 1;
     f32x4 a_ring[RING][RTILES][4];
-    // Chunk number c (0 <= c < AHEAD) counted from the start of step K-2; when NCH == 1
+    // Chunk number c (0 <= c < AHEAD) counted from the start of step r_top; when NCH == 1
     // chunk 1 is already in the next step.
 #pragma unroll
     for (int c = 0; c < AHEAD; ++c) {
-        const int rr = (K - 2) - c / NCH;
-        load_a(a_ring[c % RING], a_lane + (size_t)(rr > 0 ? rr : 0) * D * D + (c % NCH) * 32);
+        const int rr = r_top - c / NCH;
+        load_a(a_ring[c % RING], a_lane + (size_t)(rr > r_lo ? rr : r_lo) * a_stride + (c % NCH) * 32);
     }
 
     int cur = 0;
-    for (int r = K - 2; r >= 0; r -= (NCH == 1 ? 2 : 1)) {
+    for (int r = r_top; r >= r_lo; r -= (NCH == 1 ? 2 : 1)) {
         // NCH == 1 runs two steps per trip so ring indices stay compile-time constants.
 #pragma unroll
         for (int sub = 0; sub < (NCH == 1 ? 2 : 1); ++sub) {
         const int rs = r - sub;
-        if (rs < 0) break;
+        if (rs < r_lo) break;
         f32x16 acc[RTILES][CTILES];
 #pragma unroll
         for (int i = 0; i < RTILES; ++i)
@@ -158,10 +242,10 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
         float vdot[RTILES];
 #pragma unroll
         for (int i = 0; i < RTILES; ++i) vdot[i] = 0.0f;
-        const Tin* a_r = a_lane + (size_t)rs * D * D;
-        // Chunks past the end of this step belong to mats[rs-1] (a harmless re-read of
-        // mats[0] after the very last step).
-        const Tin* a_wrap = a_lane + (size_t)(rs > 0 ? rs - 1 : 0) * D * D;
+        const Tin* a_r = a_lane + (size_t)rs * a_stride;
+        // Chunks past the end of this step belong to the next step's matrix (a harmless re-read of
+        // the last one after the very last step).
+        const Tin* a_wrap = a_lane + (size_t)(rs > r_lo ? rs - 1 : r_lo) * a_stride;
 #pragma unroll
         for (int kc = 0; kc < NCH; ++kc) {
             const int slot = (NCH == 1 ? sub : kc) % RING;
@@ -212,7 +296,9 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        float* o_r = out_b + (size_t)rs * D * D;
+        // A chunk that only forms its total parks it one slot above its first matrix (phase 1).
+        const bool store = store_all || rs == r_lo;
+        float* o_r = o_base + (size_t)(store_all ? rs : rs + 1) * o_stride;
         float* st_new = lds + (cur ^ 1) * (CB * PITCH);
 #pragma unroll
         for (int i = 0; i < RTILES; ++i)
@@ -225,8 +311,10 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                     f32x4 v4 = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
                                 acc[i][j][4 * g + 3]};
                     *reinterpret_cast<f32x4*>(st_new + col * PITCH + row) = v4;
+                    if (store) {
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) o_r[(size_t)(row + t) * D + c0 + col] = v4[t];
+                        for (int t = 0; t < 4; ++t) o_r[(size_t)(row + t) * D + c0 + col] = v4[t];
+                    }
                 }
         if (COT) {
             float* v_new = vbuf + (cur ^ 1) * D;
@@ -236,7 +324,7 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 const float total = vdot[i] + __shfl_xor(vdot[i], 32, 64);  // the two k halves of a row
                 if (h == 0) {
                     v_new[row0 + i * 32 + m] = total;
-                    if (c0 == 0) cot_r[row0 + i * 32 + m] = total;
+                    if (c0 == 0 && cot_on) cot_r[row0 + i * 32 + m] = total;
                 }
             }
         }
@@ -611,26 +699,45 @@ __global__ __launch_bounds__(512) void cotangent256_half_kernel(const Tin* __res
     }
 }
 
-template <typename Tin, int D, int RT, int CB, bool COT>
-int launch_mfma_cot(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
+// cot[b, r] = out[b, r] @ g[b] for every finished suffix product (r = K is the identity: cot[b, K] = g[b]): the
+// cotangents of the K-parallel scan, whose chunks have no common chain to carry them.  One workgroup per
+// (b, r), a wave per row at a time, lanes along k (16-byte loads), butterfly fold.  d a multiple of 4.
+__global__ __launch_bounds__(256) void suffix_apply_kernel(const float* __restrict__ out, const float* __restrict__ g,
+                                                           float* __restrict__ cot, int K, int d) {
+    const int b = blockIdx.x / (K + 1);
+    const float* mat = out + (size_t)blockIdx.x * d * d;
+    const float* g_b = g + (size_t)b * d;
+    float* cot_r = cot + (size_t)blockIdx.x * d;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int row = wave; row < d; row += 4) {
+        float acc = 0.0f;
+        for (int k = lane * 4; k < d; k += 256) {
+            const f32x4 a4 = *reinterpret_cast<const f32x4*>(mat + (size_t)row * d + k);
+            const f32x4 v4 = *reinterpret_cast<const f32x4*>(g_b + k);
+            acc = fmaf(a4[0], v4[0], acc);
+            acc = fmaf(a4[1], v4[1], acc);
+            acc = fmaf(a4[2], v4[2], acc);
+            acc = fmaf(a4[3], v4[3], acc);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (lane == 0) cot_r[row] = acc;
+    }
+}
+
+template <typename Tin, int D, int RT, int CB, bool COT, int MODE = 0>
+int launch_mfma_cot(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream,
+                    ScanPlan plan = ScanPlan{0, 0, 0}) {
     constexpr int NW = D / RT;
     constexpr int NB = D / CB;
     constexpr size_t lds_bytes = ((size_t)2 * CB * (D + 4) + (COT ? 2 * D : 0)) * sizeof(float);
-    auto kern = scan_mfma_kernel<Tin, D, RT, CB, COT>;
-    if (lds_bytes > 64 * 1024) {
-        static thread_local bool attr_done[16] = {};
-        int dev = 0;
-        LBI_HIP_CHECK(hipGetDevice(&dev));
-        if (dev >= 16 || !attr_done[dev]) {
-            LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-            if (dev < 16) attr_done[dev] = true;
-        }
-    }
-    const int groups = (B + 7) / 8;
-    const dim3 grid(groups * 8 * NB);
+    auto kern = scan_mfma_kernel<Tin, D, RT, CB, COT, MODE>;
+    if (int rc = ensure_dynamic_lds<&scan_mfma_kernel<Tin, D, RT, CB, COT, MODE>>(lds_bytes)) return rc;
+    // chains in this launch (the kernel derives the same number from the plan)
+    const int chains = B * (MODE == 1 ? plan.C - 1 : 1);
+    const dim3 grid(chains >= 8 ? ((chains + 7) / 8) * 8 * NB : chains * NB);
     hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds_bytes, stream, static_cast<const Tin*>(mats),
-                       static_cast<float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), B, K);
+                       static_cast<float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), B, K, plan);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
@@ -639,6 +746,51 @@ template <typename Tin, int D, int RT, int CB>
 int launch_mfma(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream) {
     return cot ? launch_mfma_cot<Tin, D, RT, CB, true>(mats, out, g, cot, B, K, stream)
                : launch_mfma_cot<Tin, D, RT, CB, false>(mats, out, nullptr, nullptr, B, K, stream);
+}
+
+// Chunking of the K-parallel scan: C chunks of L matrices.  The dependent depth is 2L + C - 3 steps, least at
+// L ~ sqrt(K / 2).  The chunked form does twice the products, which is free only while the plain form (B * nb
+// workgroups) leaves at least half of the 256 CUs idle; C is capped so that the widest phase stays within two
+// workgroups per CU.  Measured at K = 128 (plain -> chunked, ms): d = 256: B = 1: 2.36 -> 0.28, 8: 2.04 -> 0.58,
+// 16: 2.05 -> 1.05, 32: 2.07 -> 1.8-2.1 (not taken); d = 128: B = 16: 0.35 -> 0.21, 48: 0.43 -> 0.57 (not taken).
+// Returns false when the plain chain is at least as good.  LBI_SCAN_CHUNK=0 forces the plain chain, n >= 2 chunks of n.
+inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
+    static const int forced = std::getenv("LBI_SCAN_CHUNK") ? std::atoi(std::getenv("LBI_SCAN_CHUNK")) : -1;
+    if (forced == 0) return false;
+    const int cmax = 512 / (B * nb) + 1;
+    if (K < 12 || ((B * nb > 128 || cmax < 4) && forced <= 0)) return false;
+    int L = 2;
+    while (2 * (L + 1) * (L + 1) <= K) ++L;  // floor(sqrt(K / 2))
+    if (forced > 0) L = forced < 2 ? 2 : forced;
+    int C = (K + L - 1) / L;
+    if (C > cmax && forced <= 0) {
+        L = (K + cmax - 1) / cmax;
+        C = (K + L - 1) / L;
+    }
+    if (C < 4) return false;
+    plan->L = L;
+    plan->C = C;
+    return true;
+}
+
+// The three phases of ScanPlan, one launch each on `stream` (they depend on each other in that order), then the
+// cotangents from the finished products.
+template <typename Tin, int D, int RT, int CB>
+int launch_chunked(const void* mats, void* out, const void* g, void* cot, int B, int K, ScanPlan plan,
+                   hipStream_t stream) {
+    for (int phase = 1; phase <= 3; ++phase) {
+        plan.phase = phase;
+        const int rc = phase == 2  // operands and results are fp32 products inside `out`
+                           ? launch_mfma_cot<float, D, RT, CB, false, 2>(out, out, nullptr, nullptr, B, K, stream, plan)
+                           : launch_mfma_cot<Tin, D, RT, CB, false, 1>(mats, out, nullptr, nullptr, B, K, stream, plan);
+        if (rc) return rc;
+    }
+    if (cot) {
+        hipLaunchKernelGGL(suffix_apply_kernel, dim3((unsigned)(B * (K + 1))), dim3(256), 0, stream,
+                           static_cast<const float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), K, D);
+        LBI_HIP_CHECK(hipGetLastError());
+    }
+    return LBI_OK;
 }
 
 template <typename Tin>
@@ -651,6 +803,24 @@ constexpr int kWideBlockBatch = 512;
 // other widths run the generic scan followed by the cotangent chain kernel.
 template <typename Tin>
 int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, int K, int d, hipStream_t stream) {
+    // Few batch elements: one chain per column block leaves most of the chip idle for K - 1 dependent steps, so
+    // the chain is cut into chunks that run side by side (ScanPlan), on narrow column blocks (short steps).
+    ScanPlan plan{0, 0, 0};
+    switch (d) {
+        case 256:
+            if (plan_chunks(B, K, 8, &plan)) return launch_chunked<Tin, 256, 32, 32>(mats, out, g, cot, B, K, plan, stream);
+            break;
+        case 128:
+            if (plan_chunks(B, K, 4, &plan)) return launch_chunked<Tin, 128, 32, 32>(mats, out, g, cot, B, K, plan, stream);
+            break;
+        case 64:
+            if (plan_chunks(B, K, 2, &plan)) return launch_chunked<Tin, 64, 32, 32>(mats, out, g, cot, B, K, plan, stream);
+            break;
+        case 32:
+            if (plan_chunks(B, K, 1, &plan)) return launch_chunked<Tin, 32, 32, 32>(mats, out, g, cot, B, K, plan, stream);
+            break;
+        default: break;
+    }
     switch (d) {
         case 256: {
             // bf16 storage runs on the 16-bit matrix pipes: the running suffix enters each product as bf16
@@ -734,9 +904,7 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
     if (d % per_piece == 0 && matrix_bytes <= 128 * 1024 && d / per_piece <= 64) {
         const size_t staged_bytes = matrix_bytes + (size_t)2 * d * sizeof(float);  // <= 130 KB
         auto kern = cotangent_staged_kernel<Tin>;
-        if (staged_bytes > 64 * 1024)
-            LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)staged_bytes));
+        if (int rc = ensure_dynamic_lds<&cotangent_staged_kernel<Tin>>(staged_bytes)) return rc;
         hipLaunchKernelGGL(kern, dim3(B), dim3(256), staged_bytes, stream, static_cast<const Tin*>(mats),
                            static_cast<const float*>(g), static_cast<float*>(out), K, d);
         LBI_HIP_CHECK(hipGetLastError());

@@ -227,14 +227,7 @@ __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __res
 template <int NP>
 int launch_planes(const void* mats, void* out, int B, int K, hipStream_t stream) {
     auto kern = scan_colsplit_kernel<NP>;
-    static bool attr_done[16] = {};
-    int dev = 0;
-    LBI_HIP_CHECK(hipGetDevice(&dev));
-    if (dev >= 16 || !attr_done[dev]) {
-        LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          LDS_BYTES));
-        if (dev < 16) attr_done[dev] = true;
-    }
+    if (int rc = ensure_dynamic_lds<&scan_colsplit_kernel<NP>>(LDS_BYTES)) return rc;
     const dim3 grid(((B + 7) / 8) * 8 * NB);
     hipLaunchKernelGGL(kern, grid, dim3(NT), LDS_BYTES, stream, static_cast<const bf16_raw*>(mats),
                        static_cast<float*>(out), B, K);

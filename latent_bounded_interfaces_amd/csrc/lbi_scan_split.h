@@ -279,14 +279,12 @@ int launch_planes(const void* mats, void* out, const void* g, void* cot, int B, 
     const dim3 grid(((B + 7) / 8) * 8 * NB);
     if (cot) {
         auto kern = scan_split_kernel<Tin, true, NP>;
-        LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)lds_bytes));
+        if (int rc = ensure_dynamic_lds<&scan_split_kernel<Tin, true, NP>>(lds_bytes)) return rc;
         hipLaunchKernelGGL(kern, grid, dim3(NT), lds_bytes, stream, static_cast<const Tin*>(mats),
                            static_cast<float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), B, K);
     } else {
         auto kern = scan_split_kernel<Tin, false, NP>;
-        LBI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)lds_bytes));
+        if (int rc = ensure_dynamic_lds<&scan_split_kernel<Tin, false, NP>>(lds_bytes)) return rc;
         hipLaunchKernelGGL(kern, grid, dim3(NT), lds_bytes, stream, static_cast<const Tin*>(mats),
                            static_cast<float*>(out), static_cast<const float*>(nullptr), static_cast<float*>(nullptr),
                            B, K);

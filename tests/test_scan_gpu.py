@@ -211,6 +211,91 @@ def test_benchmark_shape_properties(device):
     assert _rel_err(out_bf16[pick].cpu(), truth_bf) <= BF16_D256_BAR
 
 
+@pytest.mark.parametrize("bsz", [1, 2, 4, 8])
+@pytest.mark.parametrize("kind", ["near_identity", "randn"])
+def test_k_parallel_scan_at_small_batches(bsz, kind, device):
+    """K=128, d=256 with so few batch elements that the chain is cut into chunks that run side by side
+    (three launches): same results as the sequential product to the fp32 bar, identity tail, cotangents,
+    reruns bit-identical, fused entry == matrices-only entry."""
+    from latent_bounded_interfaces_amd.hip.interface import (suffix_scan_pullbacks,
+                                                             suffix_scan_pullbacks_and_cotangents)
+
+    count, rank = 128, 256
+    mats, g = oscan.make_scan_inputs(bsz, count, rank, kind=kind, seed=7)
+    mats_d, g_d = mats.to(device), g.to(device)
+    out = suffix_scan_pullbacks(mats_d)
+    assert torch.equal(out, suffix_scan_pullbacks(mats_d)), "reruns differ"
+    assert torch.equal(out[:, count], torch.eye(rank, device=device).expand(bsz, rank, rank))
+    assert torch.equal(out[:, count - 1], mats_d[:, count - 1])
+    truth = oscan.suffix_scan_sequential(mats, dtype=torch.float64)
+    assert _rel_err(out.cpu(), truth) <= 1e-5
+    fused, cot = suffix_scan_pullbacks_and_cotangents(mats_d, g_d)
+    assert torch.equal(fused, out)
+    assert torch.equal(cot[:, count].cpu(), g)
+    want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+    scale = want.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+    assert float(((cot.cpu().double() - want).abs() / scale).max()) <= 1e-5
+    again = suffix_scan_pullbacks_and_cotangents(mats_d, g_d)
+    assert torch.equal(again[0], fused) and torch.equal(again[1], cot)
+
+
+# chains long enough to be cut, at every matrix-core width the chunked form runs, lengths that leave a ragged or
+# one-matrix last chunk, batch sizes either side of the 8-chain launch mapping
+K_PARALLEL_SHAPES = [(1, 13, 32), (1, 37, 64), (2, 100, 128), (3, 61, 256), (1, 12, 256), (1, 129, 256), (9, 33, 32),
+                     (7, 50, 64), (2, 17, 100), (1, 40, 200)]
+
+
+@pytest.mark.parametrize("shape", K_PARALLEL_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_k_parallel_scan_shapes(shape, dtype, device):
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks_and_cotangents
+
+    bsz, count, rank = shape
+    mats, g = oscan.make_scan_inputs(bsz, count, rank, kind="randn", seed=8)
+    mats = mats.to(dtype)
+    out, cot = suffix_scan_pullbacks_and_cotangents(mats.to(device), g.to(device))
+    truth = oscan.suffix_scan_sequential(mats.float(), dtype=torch.float64)
+    assert torch.equal(out[:, count].cpu(), torch.eye(rank).expand(bsz, rank, rank))
+    assert _rel_err(out.cpu(), truth) <= 1e-5
+    # The chunks share no chain, so these cotangents are the finished products applied to g, which is how the
+    # reference gets them (backward/suffix_scan.py:49-53): the 1e-5 of a product can be amplified where the
+    # mat-vec cancels, hence 3e-5 per vector here, and the reference's own bar for this quantity, an RMS
+    # difference to the sequential chain below 1e-5 (backward/scan.py:63-72, tests/test_lbi_gradient_parity.py:44).
+    want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+    scale = want.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+    assert float(((cot.cpu().double() - want).abs() / scale).max()) <= 3e-5
+    assert float(torch.sqrt((((cot.cpu().double() - want) / scale) ** 2).mean())) <= 1e-5
+
+
+@pytest.mark.parametrize("chunk", [0, 2, 3, 5, 16])
+def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, device):
+    """LBI_SCAN_CHUNK forces the chunk length (0: the plain chain): every cut of K=13 / 33 / 64, including a
+    one-matrix last chunk, meets the bar, with and without the cotangent chain."""
+    import os
+    import subprocess
+    import sys
+
+    code = (
+        "import torch, sys; sys.path.insert(0, %r);"
+        "from oracle import scan as o;"
+        "from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks as s, "
+        "suffix_scan_pullbacks_and_cotangents as f;"
+        "worst = 0.0\n"
+        "for shape in ((1, 13, 64), (2, 33, 256), (1, 64, 32), (3, 21, 128)):\n"
+        "    m, g = o.make_scan_inputs(*shape, kind='randn', seed=5)\n"
+        "    t = o.suffix_scan_sequential(m, dtype=torch.float64)\n"
+        "    c = o.suffix_cotangents_sequential(m.double(), g.double())\n"
+        "    out, cot = f(m.cuda(), g.cuda())\n"
+        "    assert torch.equal(out, s(m.cuda()))\n"
+        "    worst = max(worst, float(((out.cpu().double() - t).abs().flatten(2).amax(2) / t.abs().flatten(2).amax(2)).max()))\n"
+        "    worst = max(worst, float(((cot.cpu().double() - c).abs() / c.abs().amax(2, keepdim=True)).max()))\n"
+        "print(worst); sys.exit(0 if 0.0 < worst <= 1e-5 else 1)"
+    ) % str(Path(__file__).resolve().parents[1])
+    env = dict(os.environ, LBI_SCAN_CHUNK=str(chunk))
+    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stdout + res.stderr
+
+
 def test_backward_module_contract(device):
     """Counterpart functions of reference backward/suffix_scan.py keep its edge cases."""
     from latent_bounded_interfaces_amd.backward import suffix_scan as bs
