@@ -34,11 +34,13 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 
 SCAN_B, SCAN_K, SCAN_D = 64, 128, 256
 
-# HBM bytes per launch of the scan kernel at this shape, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 1 GiB device
-# copy (FETCH_SIZE reads 0.5 KiB per KiB moved on this part, WRITE_SIZE 1.0):
-# 1 052 300 KiB * 2.0 + 2 121 792 KiB * 1.0.  See profiles/scan_fp32_B64_K128_d256_pmc.md.
-MEASURED_SCAN_TRAFFIC_BYTES = int((1052300 * 2.0 + 2121792 * 1.0) * 1024)
+# HBM bytes per launch of the scan kernel at this shape come from a small JSON beside the counter summary in
+# profiles/ (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, KiB per dispatch, each scaled by the same counter's
+# reading for a 1 GiB device copy).  The file names the kernel and carries a hash of the kernel's sources; when
+# either no longer matches, the line reports "traffic": null rather than a figure measured on other code.
+SCAN_KERNEL = "scan_mfma_kernel<float, 256, 32, 64, true, 0>"
+SCAN_TRAFFIC_JSON = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                                 "scan_fp32_B64_K128_d256_pmc.json")
 
 
 def _parse() -> argparse.Namespace:
@@ -164,6 +166,7 @@ def main() -> int:
     torch.cuda.set_device(device)
 
     from latent_bounded_interfaces_amd import _lib
+    from latent_bounded_interfaces_amd import benchmarks as lbi_bench
 
     lib = _lib.load()
     stream = _lib.current_stream_ptr(device)
@@ -237,12 +240,12 @@ def main() -> int:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "scan_mfma_kernel<float,256,32,64,true> (lbi_suffix_scan_with_cotangents)",
+            "kernel": SCAN_KERNEL + " (lbi_suffix_scan_with_cotangents)",
             "achieved": achieved_tflops,
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved_tflops / PEAK_FP32_MFMA_TFLOPS,
-            "traffic": MEASURED_SCAN_TRAFFIC_BYTES,
+            "traffic": lbi_bench.load_traffic(SCAN_TRAFFIC_JSON, SCAN_KERNEL),
             "kernel_ms_avg": scan_avg,
             "kernel_ms_min": min(scan_ms),
             "algorithmic_flops": scan_flops,
@@ -286,16 +289,11 @@ def main() -> int:
                              "unit": "GB/s", "frac": bf_bytes / (bf_avg * 1e-3) / 1e9 / PEAK_HBM_GBS},
             }
         del mats_bf16
-        try:
-            from latent_bounded_interfaces_amd import benchmarks as lbi_bench
-
-            extra.update(lbi_bench.attention_section(steps=max(3, args.steps // 4)))
-            torch.cuda.empty_cache()
-            extra.update(lbi_bench.region_section(steps=max(3, args.steps // 4)))
-            torch.cuda.empty_cache()
-            extra.update(lbi_bench.lbi_step_section(steps=3))
-        except ImportError:
-            pass
+        extra.update(lbi_bench.attention_section(steps=max(3, args.steps // 4)))
+        torch.cuda.empty_cache()
+        extra.update(lbi_bench.region_section(steps=max(3, args.steps // 4)))
+        torch.cuda.empty_cache()
+        extra.update(lbi_bench.lbi_step_section(steps=3))
         result["extra"] = extra
 
     if not args.no_cpu_baseline:

@@ -2,19 +2,24 @@
 
 Counterpart of reference benchmarks/time_attention_pullback.py: warm-up, then the
 median and best of ``iters`` device-timed calls (HIP events on the launch stream,
-reference :117-138), the same CSV columns (reference :347-360), an optional error
-check against a caller-supplied expected result.  ``attention_section`` is what
-``bench.py`` embeds: the long-context and the reference benchmark shape with their
-roofline figures.
+reference :117-138), the same CSV columns (reference :347-360), and its ``--check``
+(:230, :300-305): the result compared with one SDPA forward + autograd backward per
+direction, in fp32 on the device, on a bounded sample of (batch, head) pairs and
+directions.  ``attention_section`` is what ``bench.py`` embeds: the long-context and the
+reference benchmark shape with their roofline figures.  ``--pmc-traffic`` turns two
+``rocprofv3 --pmc`` counter dumps into the small JSON ``bench.py`` reads its HBM traffic
+figure from.
 """
 from __future__ import annotations
 
 import argparse
 import csv
+import hashlib
 import json
 import math
 import statistics
 import sys
+from pathlib import Path
 
 import torch
 
@@ -89,7 +94,33 @@ def time_call(fn, *, warmup: int, iters: int):
     return statistics.median(times), min(times), statistics.fmean(times), peak
 
 
-def measure(B, H, T, Dh, P, dtype, *, causal=True, warmup=3, iters=10, device="cuda", expected=None):
+def check_against_autograd(outputs, q, k, v, g, scale: float, causal: bool, *, pairs: int = 2, directions: int = 2):
+    """What the reference benchmark's ``--check`` computes (benchmarks/time_attention_pullback.py:300-305): the
+    largest absolute difference to per-direction SDPA + autograd, here in fp32 on the device and on a bounded
+    sample: the first and last ``pairs`` (batch, head) pairs and the first and last ``directions`` directions (all of
+    them when the call is small).  Returns ``(max_abs_error, max_abs_error / max|expected|, sample description)``."""
+    B, H, T, Dh = q.shape
+    P = g.shape[1]
+    flat = list(range(B * H))
+    picked = sorted(set(flat[:pairs] + flat[-pairs:]))
+    dirs = sorted(set(list(range(P))[:directions] + list(range(P))[-directions:]))
+    worst, largest = 0.0, 0.0
+    for bh in picked:
+        b, h = divmod(bh, H)
+        qs, ks, vs = (t[b:b + 1, h:h + 1].float().detach().requires_grad_(True) for t in (q, k, v))
+        with torch.enable_grad():
+            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, is_causal=causal, scale=scale)
+            for p in dirs:
+                want = torch.autograd.grad(out, (qs, ks, vs), grad_outputs=g[b:b + 1, p, h:h + 1].float(),
+                                           retain_graph=True)
+                for got, ref in zip(outputs, want):
+                    worst = max(worst, float((got[b, p, h].float() - ref[0, 0]).abs().max()))
+                    largest = max(largest, float(ref.abs().max()))
+    sample = f"{len(picked)} of {B * H} (batch, head) pairs x {len(dirs)} of {P} directions, fp32 SDPA + autograd on the device"
+    return worst, worst / max(largest, 1e-30), sample
+
+
+def measure(B, H, T, Dh, P, dtype, *, causal=True, warmup=3, iters=10, device="cuda", check=False):
     q, k, v, g = make_inputs(B, H, T, Dh, P, dtype, device)
     call = PullbackCall(q, k, v, g, 1.0 / math.sqrt(Dh), causal)
     median_ms, best_ms, mean_ms, peak = time_call(call, warmup=warmup, iters=iters)
@@ -97,47 +128,98 @@ def measure(B, H, T, Dh, P, dtype, *, causal=True, warmup=3, iters=10, device="c
     again = call()
     torch.cuda.synchronize()
     stable = all(torch.equal(a, b) for a, b in zip(first, again))
-    err = None
-    if expected is not None:
-        err = max(float((a.float() - b.float().to(a.device)).abs().max()) for a, b in zip(first, expected))
+    err = rel_err = sample = None
+    if check:
+        err, rel_err, sample = check_against_autograd(first, q, k, v, g, 1.0 / math.sqrt(Dh), causal)
     flops = algorithmic_flops(B, H, T, Dh, P, causal)
     tflops = flops / (mean_ms * 1e-3) / 1e12
     return {
         "B": B, "H": H, "T": T, "Dh": Dh, "P": P, "causal": causal, "dtype": str(dtype).replace("torch.", ""),
         "backend": "hip", "median_ms": median_ms, "best_ms": best_ms, "mean_ms": mean_ms,
-        "peak_memory_bytes": peak, "max_abs_error_vs_autograd": err,
-        "algorithmic_flops": flops, "tflops": tflops, "bit_stable_rerun": stable,
+        "peak_memory_bytes": peak, "max_abs_error_vs_autograd": err, "max_rel_error_vs_autograd": rel_err,
+        "check_sample": sample, "algorithmic_flops": flops, "tflops": tflops, "bit_stable_rerun": stable,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_MFMA_16BIT_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_MFMA_16BIT_TFLOPS},
     }
 
 
-def graph_replay_ms(call, *, iters: int = 50) -> float:
-    """Median time of one replay of ``call`` captured into a HIP graph (the launch-bound small shapes:
-    one graph launch instead of one launch per kernel)."""
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        call()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        call()
-    median_ms, _, _, _ = time_call(graph.replay, warmup=5, iters=iters)
-    return median_ms
-
-
 def attention_section(steps: int = 5) -> dict:
-    """The two attention configurations reported beside the scan headline."""
+    """The two attention configurations reported beside the scan headline, each checked against autograd."""
     out = {}
-    out["attn_pullback_bf16_B4_H16_T4096_Dh128_P16"] = measure(4, 16, 4096, 128, 16, torch.bfloat16, iters=steps)
+    out["attn_pullback_bf16_B4_H16_T4096_Dh128_P16"] = measure(4, 16, 4096, 128, 16, torch.bfloat16, iters=steps,
+                                                               check=True)
     torch.cuda.empty_cache()
-    small = measure(8, 8, 128, 64, 4, torch.float16, iters=max(steps, 20))
-    q, k, v, g = make_inputs(8, 8, 128, 64, 4, torch.float16, "cuda")
-    small["graph_replay_ms"] = graph_replay_ms(PullbackCall(q, k, v, g, 1.0 / math.sqrt(64), True))
-    out["attn_pullback_fp16_B8_H8_T128_Dh64_P4"] = small
+    out["attn_pullback_fp16_B8_H8_T128_Dh64_P4"] = measure(8, 8, 128, 64, 4, torch.float16, iters=max(steps, 20),
+                                                           check=True)
     return out
+
+
+# ---------------------------------------------------------------------------------------
+# HBM traffic of a kernel from rocprofv3 counter dumps
+# ---------------------------------------------------------------------------------------
+PACKAGE_DIR = Path(__file__).resolve().parent
+
+
+def source_digest(files) -> str:
+    """sha256 over the named kernel sources (paths relative to the package), the tie between a measured
+    counter figure and the code it was measured on."""
+    h = hashlib.sha256()
+    for name in sorted(files):
+        h.update(name.encode())
+        h.update((PACKAGE_DIR / name).read_bytes())
+    return h.hexdigest()
+
+
+def _per_dispatch(csv_path: Path, counter: str, kernel_substring: str, *, first_only: bool = False) -> tuple[float, int]:
+    rows = []
+    with open(csv_path, newline="") as fh:
+        for row in csv.DictReader(fh):
+            if row["Counter_Name"] == counter and kernel_substring in row["Kernel_Name"]:
+                rows.append((int(row["Dispatch_Id"]), float(row["Counter_Value"])))
+    if not rows:
+        raise SystemExit(f"{csv_path}: no {counter} rows for a kernel containing {kernel_substring!r}")
+    rows.sort()
+    values = [v for _, v in rows[:1]] if first_only else [v for _, v in rows]
+    return statistics.fmean(values), len(values)
+
+
+def pmc_traffic(fetch_dir: str, write_dir: str, *, kernel: str, copy_kernel: str, copy_bytes: int, sources) -> dict:
+    """HBM bytes per dispatch of ``kernel`` from two ``rocprofv3 --pmc`` runs (FETCH_SIZE, then WRITE_SIZE, KiB per
+    dispatch), each counter scaled by what it reads for a plain device copy of ``copy_bytes`` in the same run: the
+    FIRST dispatch of ``copy_kernel``, which is where ``bench.py --copy-calibration`` puts it."""
+    def one(directory, counter):
+        path = next(Path(directory).rglob("*counter_collection.csv"))
+        value, calls = _per_dispatch(path, counter, kernel)
+        copy_value, _ = _per_dispatch(path, counter, copy_kernel, first_only=True)
+        return value, calls, copy_value
+
+    fetch, calls, copy_fetch = one(fetch_dir, "FETCH_SIZE")
+    write, _, copy_write = one(write_dir, "WRITE_SIZE")
+    fetch_scale = (copy_bytes / 1024.0) / copy_fetch
+    write_scale = (copy_bytes / 1024.0) / copy_write
+    return {
+        "kernel": kernel, "dispatches_averaged": calls,
+        "fetch_size_kib": fetch, "write_size_kib": write,
+        "copy_kernel": copy_kernel, "copy_bytes": copy_bytes,
+        "copy_fetch_size_kib": copy_fetch, "copy_write_size_kib": copy_write,
+        "fetch_scale": fetch_scale, "write_scale": write_scale,
+        "traffic_bytes": int((fetch * fetch_scale + write * write_scale) * 1024),
+        "sources": sorted(sources), "source_sha256": source_digest(sources),
+    }
+
+
+def load_traffic(json_path, kernel_substring: str):
+    """The measured traffic figure, or None when the file is missing, names another kernel, or the kernel sources
+    have changed since it was measured (the figure would describe code that no longer exists)."""
+    try:
+        record = json.loads(Path(json_path).read_text())
+        if kernel_substring not in record["kernel"] and record["kernel"] not in kernel_substring:
+            return None
+        if source_digest(record["sources"]) != record["source_sha256"]:
+            return None
+        return int(record["traffic_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 # ---------------------------------------------------------------------------------------
@@ -357,9 +439,30 @@ def main(argv=None) -> int:
     ap.add_argument("--basis", type=int, default=64, help="cotangent directions of the --region run")
     ap.add_argument("--lbi-step", action="store_true",
                     help="time the device work of one LBI scan backward step at the end-to-end configuration")
+    ap.add_argument("--check", action="store_true",
+                    help="compare with per-direction SDPA + autograd (fp32, on the device, bounded sample) and fail "
+                         "when the largest error exceeds --check-tol")
+    ap.add_argument("--check-tol", type=float, default=None,
+                    help="bound on max|error| / max|expected| (default 2e-5 for float32, 2e-2 for 16-bit storage)")
+    ap.add_argument("--pmc-traffic", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"), default=None,
+                    help="write the HBM-traffic JSON of --kernel from two rocprofv3 --pmc output folders")
+    ap.add_argument("--kernel", default="scan_mfma_kernel<float, 256, 32, 64, true, 0>")
+    ap.add_argument("--copy-kernel", default="__amd_rocclr_copyBuffer")
+    ap.add_argument("--copy-bytes", type=int, default=1 << 30)
+    ap.add_argument("--sources", nargs="*", default=["csrc/lbi_scan.hip", "csrc/lbi_common.h"])
+    ap.add_argument("--out", default=None, help="--pmc-traffic: where to write the JSON (default: stdout)")
     ap.add_argument("--scan", nargs="*", default=None, help="time the fused suffix scan instead: B,K,d tuples")
     ap.add_argument("--matrices-only", action="store_true", help="--scan: the suffix matrices without the cotangents")
     args = ap.parse_args(argv)
+    if args.pmc_traffic is not None:
+        record = pmc_traffic(*args.pmc_traffic, kernel=args.kernel, copy_kernel=args.copy_kernel,
+                             copy_bytes=args.copy_bytes, sources=args.sources)
+        text = json.dumps(record, indent=2) + "\n"
+        if args.out:
+            Path(args.out).write_text(text)
+        else:
+            sys.stdout.write(text)
+        return 0
     if args.scan is not None:
         for spec in args.scan:
             B, K, d = (int(x) for x in spec.split(","))
@@ -375,11 +478,16 @@ def main(argv=None) -> int:
                                         iters=args.iters)), flush=True)
         return 0
     rows = []
+    failed = False
+    tol = args.check_tol if args.check_tol is not None else (2e-5 if args.dtype == "float32" else 2e-2)
     for spec in args.shapes:
         B, H, T, Dh, P = (int(x) for x in spec.split(","))
         rows.append(measure(B, H, T, Dh, P, getattr(torch, args.dtype), causal=not args.non_causal,
-                            warmup=args.warmup, iters=args.iters))
+                            warmup=args.warmup, iters=args.iters, check=args.check))
         print(json.dumps(rows[-1]), flush=True)
+        if args.check and rows[-1]["max_rel_error_vs_autograd"] > tol:
+            print(f"check failed for {spec}: {rows[-1]['max_rel_error_vs_autograd']:.3e} > {tol:.1e}", file=sys.stderr)
+            failed = True
     if args.csv:
         with open(args.csv, "w", newline="") as fh:
             writer = csv.DictWriter(fh, fieldnames=CSV_COLUMNS, extrasaction="ignore")
@@ -388,7 +496,7 @@ def main(argv=None) -> int:
     if args.json:
         with open(args.json, "w") as fh:
             json.dump(rows, fh, indent=2)
-    return 0
+    return 1 if failed else 0
 
 
 if __name__ == "__main__":
