@@ -289,6 +289,7 @@ def main() -> int:
                              "unit": "GB/s", "frac": bf_bytes / (bf_avg * 1e-3) / 1e9 / PEAK_HBM_GBS},
             }
         del mats_bf16
+        extra.update(lbi_bench.scan_section(steps=max(5, args.steps // 2)))
         extra.update(lbi_bench.attention_section(steps=max(3, args.steps // 4)))
         torch.cuda.empty_cache()
         extra.update(lbi_bench.region_section(steps=max(3, args.steps // 4)))

@@ -425,6 +425,46 @@ def measure_scan(B: int, K: int, d: int, dtype, *, warmup=3, iters=10, device="c
             "algorithmic_gbs": nbytes / (median_ms * 1e-3) / 1e9, "algorithmic_bytes": nbytes}
 
 
+def measure_cotangent_chain(B: int, K: int, d: int, dtype, *, warmup=2, iters=10, device="cuda") -> dict:
+    """The cotangent-only chain (``lbi_suffix_cotangents``): one pass over the matrices, no d x d product; the
+    rate is quoted on the bytes of the matrices, which is all it has to move."""
+    lib = _lib.load()
+    gen = torch.Generator(device=device).manual_seed(0)
+    mats = torch.randn(B, K, d, d, device=device, generator=gen).mul_((0.01 / d) ** 0.5)
+    mats.diagonal(dim1=-2, dim2=-1).add_(1.0)
+    mats = mats.to(dtype)
+    g = torch.randn(B, d, device=device, generator=gen)
+    out = torch.empty(B, K + 1, d, device=device)
+
+    def call():
+        _lib.check(lib.lbi_suffix_cotangents(mats.data_ptr(), g.data_ptr(), out.data_ptr(), B, K, d,
+                                             _lib.dtype_code(mats.dtype), _lib.current_stream_ptr(mats.device)),
+                   "lbi_suffix_cotangents")
+
+    median_ms, best_ms, mean_ms, _ = time_call(call, warmup=warmup, iters=iters)
+    nbytes = float(mats.numel() * mats.element_size())
+    gbs = nbytes / (mean_ms * 1e-3) / 1e9
+    return {"B": B, "K": K, "d": d, "dtype": str(dtype).replace("torch.", ""), "kernel_ms_avg": mean_ms,
+            "best_ms": best_ms, "pullbacks_per_s": B * K / (mean_ms * 1e-3),
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0}}
+
+
+def scan_section(steps: int = 10) -> dict:
+    """Scan variants beside the headline: the cotangent-only chain at a batch that gives every CU a batch element
+    (one workgroup runs one chain), and the K-parallel form of the scan at the batch sizes the reference's own
+    tests and paper launcher use (one to a few elements)."""
+    out = {}
+    for dtype, tag in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+        out[f"scan_cotangent_only_{tag}_B256"] = measure_cotangent_chain(256, 128, 256, dtype, iters=steps)
+        torch.cuda.empty_cache()
+    for batch in (1, 8):
+        row = measure_scan(batch, 128, 256, torch.float32, iters=steps)
+        row["roofline"] = {"bound": "mfma", "achieved": row["tflops"], "peak": 157.3, "unit": "TFLOP/s",
+                           "frac": row["tflops"] / 157.3}
+        out[f"scan_kparallel_fp32_B{batch}_K128_d256"] = row
+    return out
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.splitlines()[0])
     ap.add_argument("--shapes", nargs="*", default=["1,8,128,64,4"], help="B,H,T,Dh,P tuples")
