@@ -77,7 +77,8 @@ class StructuredInterfacePullbackProvider:
             return first if flags[0] else g_region_output
         return first if bool(torch.equal(first, g_region_output)) else g_region_output
 
-    def region_state_jacobian_t(self, *, model: Any, region_cache: Any) -> torch.Tensor:
+    def region_state_jacobian_t(self, *, model: Any, region_cache: Any, out: torch.Tensor | None = None) -> torch.Tensor:
+        """``Jt`` of one region, ``[B, d, d]``; written into ``out`` (any strides) when given."""
         state_in = region_cache.state_in
         if state_in.dim() != 2:
             raise ValueError("interface state inputs must be [B, R].")
@@ -96,14 +97,32 @@ class StructuredInterfacePullbackProvider:
                 decode = model.interface.apply_decode_jacobian_t_to_state_input(
                     region_cache=region_cache, region_input_cotangent_basis=g_region_input)
                 total = update["g_state_skip"] + decode["g_state_input"]  # [B, P, d_in]
-                cols.append(total.transpose(1, 2))                        # [B, d_in, P]
+                if out is not None:
+                    out[:, :, start:start + total.shape[1]].copy_(total.transpose(1, 2))
+                else:
+                    cols.append(total.transpose(1, 2))                    # [B, d_in, P]
+        if out is not None:
+            return out
         return torch.cat(cols, dim=-1).to(device=state_in.device, dtype=state_in.dtype).contiguous()
 
     def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
+        """One ``[B, d, d]`` tensor per region.  The first K - 1 of them are slices of ONE dense ``[B, K-1, d, d]``
+        buffer, in order: the scan backward step composes exactly those (the last region's output state never
+        reaches the loss, reference backward/suffix_scan.py:71), and ``backward.suffix_scan`` hands such a list to
+        the kernels as it lies, without the stacking copy (reference backward/suffix_scan.py:17)."""
         region_caches = cache["region_caches"]
-        if len(region_caches) != model.num_regions:
+        count = len(region_caches)
+        if count != model.num_regions:
             raise ValueError("cache has invalid region_caches length.")
-        return [self.region_state_jacobian_t(model=model, region_cache=rc) for rc in region_caches]
+        if count < 2:
+            return [self.region_state_jacobian_t(model=model, region_cache=rc) for rc in region_caches]
+        state = region_caches[0].state_in
+        bsz, rank = state.shape
+        inner = torch.empty((bsz, count - 1, rank, rank), device=state.device, dtype=state.dtype)
+        result = [self.region_state_jacobian_t(model=model, region_cache=rc, out=inner[:, r])
+                  for r, rc in enumerate(region_caches[:-1])]
+        result.append(self.region_state_jacobian_t(model=model, region_cache=region_caches[-1]))
+        return result
 
 
 class TorchGraphInterfacePullbackProvider:

@@ -25,7 +25,7 @@ def compose_suffix_jacobian_t(state_jacobians_t: Sequence[torch.Tensor]) -> list
     bsz, rank, rank2 = state_jacobians_t[0].shape
     if rank != rank2:
         raise ValueError("interface state Jacobian-transpose tensors must be square.")
-    stacked = torch.stack(list(state_jacobians_t), dim=1).contiguous()
+    stacked = _stack_for_chain(state_jacobians_t)
     suffix = suffix_scan_jacobian_t(stacked)
     if suffix.shape != (bsz, count + 1, rank, rank):
         raise ValueError("suffix scan returned an unexpected shape")
@@ -56,10 +56,34 @@ def apply_jacobian_t(
     return chain[:, 0].to(device=cotangent.device, dtype=out_dtype)
 
 
+def _dense_stack_view(mats: Sequence[torch.Tensor]) -> torch.Tensor | None:
+    """The list as one ``[B, K, d, d]`` tensor WITHOUT a copy, if its members are, in order, the K slices
+    ``buf[:, r]`` of one dense ``[B, K, d, d]`` buffer (what ``StructuredInterfacePullbackProvider`` returns for
+    the matrices the scan composes); else None."""
+    first = mats[0]
+    count = len(mats)
+    bsz, rank, _ = first.shape
+    item, step = first.element_size(), rank * rank
+    want_strides = (count * step, rank, 1)
+    for r, m in enumerate(mats):
+        if (m.shape != first.shape or m.dtype != first.dtype or m.device != first.device
+                or (bsz > 1 and m.stride() != want_strides) or m.stride()[1:] != want_strides[1:]
+                or m.data_ptr() != first.data_ptr() + r * step * item
+                or m.untyped_storage().data_ptr() != first.untyped_storage().data_ptr()):
+            return None
+    need = first.storage_offset() + (bsz - 1) * count * step + count * step
+    if first.untyped_storage().nbytes() < need * item:
+        return None
+    return torch.as_strided(first, (bsz, count, rank, rank), (count * step, step, rank, 1))
+
+
 def _stack_for_chain(state_jacobians_t: Sequence[torch.Tensor]) -> torch.Tensor:
     bsz, rank, rank2 = state_jacobians_t[0].shape
     if rank != rank2:
         raise ValueError("interface state Jacobian-transpose tensors must be square.")
+    dense = _dense_stack_view(state_jacobians_t)
+    if dense is not None:
+        return dense
     return torch.stack(list(state_jacobians_t), dim=1).contiguous()
 
 

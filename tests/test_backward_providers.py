@@ -103,3 +103,26 @@ def test_grad_map_helpers_round_trip():
     result = backward.ADResult(grad_map={})
     assert result.diagnostics == {}
     assert backward.LBIBackwardResult(grad_map={}, interface_scan_rms=0.5).interface_jacobian_stats is None
+
+
+def test_slices_of_one_buffer_are_recognised_without_a_copy():
+    """Lists whose members are, in order, the slices of one dense [B, K, d, d] buffer reach the kernels as that
+    buffer; anything else (separate tensors, wrong order, a gap, other strides) takes the stacking copy."""
+    from latent_bounded_interfaces_amd.backward.suffix_scan import _dense_stack_view
+
+    buf = torch.randn(3, 4, 5, 5)
+    views = [buf[:, r] for r in range(4)]
+    dense = _dense_stack_view(views)
+    assert dense is not None and dense.data_ptr() == buf.data_ptr() and dense.is_contiguous()
+    assert torch.equal(dense, buf)
+    assert _dense_stack_view([v.clone() for v in views]) is None
+    assert _dense_stack_view(views[::-1]) is None
+    assert _dense_stack_view(views[:3]) is None                      # a prefix has the wrong batch stride
+    assert _dense_stack_view([views[0], views[2]]) is None
+    assert _dense_stack_view([buf[:, r].transpose(1, 2) for r in range(4)]) is None
+    inner = buf[:, 1:3]                                              # a window of a larger buffer is not dense
+    assert _dense_stack_view([inner[:, 0], inner[:, 1]]) is None
+    one = torch.randn(1, 2, 3, 3)                                    # B = 1: the batch stride is immaterial
+    assert torch.equal(_dense_stack_view([one[:, 0], one[:, 1]]), one)
+    offset = torch.randn(2 * 3 * 4 * 4 + 7)[7:].view(2, 3, 4, 4)     # a buffer that starts inside its storage
+    assert torch.equal(_dense_stack_view([offset[:, r] for r in range(3)]), offset)

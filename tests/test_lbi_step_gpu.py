@@ -29,8 +29,15 @@ def test_structured_jacobians_match_graph_provider(basis_chunk, device):
     got = StructuredInterfacePullbackProvider(basis_chunk=basis_chunk).materialize_state_jacobian_t(model=model, cache=cache)
     assert len(got) == len(want) == 3
     for a, b in zip(got, want):
-        assert a.shape == b.shape == (2, 8, 8) and a.is_contiguous()
+        assert a.shape == b.shape == (2, 8, 8)
         assert float((a - b).abs().max()) <= 2e-5 * float(b.abs().max()), float((a - b).abs().max())
+    # the matrices the scan composes (all but the last) are slices of one dense buffer and reach the kernels as
+    # that buffer, without a stacking copy
+    from latent_bounded_interfaces_amd.backward.suffix_scan import _stack_for_chain
+
+    stacked = _stack_for_chain(got[:-1])
+    assert stacked.shape == (2, 2, 8, 8) and stacked.is_contiguous() and stacked.data_ptr() == got[0].data_ptr()
+    assert got[-1].is_contiguous()
 
 
 def test_position_constant_update_is_detected_and_optional(device):
