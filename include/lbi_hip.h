@@ -87,6 +87,19 @@ int lbi_suffix_cotangents(const void* mats, const void* g, void* out,
                           int in_dtype, void* stream);
 
 /*
+ * Suffix matrices applied to the terminal cotangent, all of them in one launch:
+ *
+ *   suffix [B, M, d, d] (fp32), g [B, d] (fp32)  ->  out [B, M, d] (fp32),   out[b, r] = suffix[b, r] @ g[b]
+ *
+ * The K mat-vecs apply_jacobian_t(suffix[r], g) of propagate_state_adjoint_with_jacobian_scan in the reference
+ * (backward/suffix_scan.py:49-53, :24-38), on the result of lbi_suffix_scan (M = K + 1 covers the identity tail,
+ * which returns g itself).  With the chain cotangents of lbi_suffix_scan_with_cotangents it gives the two sides of
+ * the reference's per-step cross-check interface_scan_rms (backward/scan.py:63-72).
+ */
+int lbi_suffix_apply(const void* suffix, const void* g, void* out,
+                     int64_t B, int64_t M, int64_t d, void* stream);
+
+/*
  * Attention input-pullback for P cotangent basis directions at once.
  *
  *   q, k, v [B, H, T, Dh],  d_out [B, P, H, T, Dh]   (dtype)

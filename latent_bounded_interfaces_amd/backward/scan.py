@@ -22,7 +22,7 @@ from typing import Any
 import torch
 from torch import nn
 
-from ..hip.interface import suffix_scan_cotangents, suffix_scan_pullbacks_and_cotangents
+from ..hip.interface import suffix_apply, suffix_scan_pullbacks_and_cotangents
 from .base import ADResult, LBIBackwardResult, ScanBackpropModel, assign_grad_map
 from .local_vjp import TorchAutogradLocalVJPProvider
 from .pullbacks import build_interface_pullback_provider
@@ -36,14 +36,12 @@ from .suffix_scan import (
 def _adjoints_and_scan_rms(state_jacobians_t, g_last_input: torch.Tensor) -> tuple[list[torch.Tensor], float]:
     """State adjoints of every region input plus the RMS difference between the two ways of getting them."""
     stacked = _stack_for_chain(state_jacobians_t[:-1])            # the last region's output state is unused
-    bsz, count, rank, _ = stacked.shape
+    count = stacked.shape[1]
     suffix, chain = suffix_scan_pullbacks_and_cotangents(stacked, g_last_input)
-    g32 = g_last_input.to(device=stacked.device, dtype=torch.float32)
-    # suffix[b, r] @ g[b] for all (b, r) at once: B*count one-step chains
-    applied = suffix_scan_cotangents(suffix[:, :count].reshape(bsz * count, 1, rank, rank),
-                                     g32.repeat_interleave(count, dim=0))[:, 0].reshape(bsz, count, rank)
-    # mean over the count + 1 regions of the per-region mean square; the last region's entry is g in both lists
-    rms = torch.sqrt(((applied - chain[:, :count]) ** 2).sum() / float(bsz * (count + 1) * rank))
+    # suffix[b, r] @ g[b] for all (b, r) at once (the identity tail returns g, as the chain does)
+    applied = suffix_apply(suffix, g_last_input)
+    # mean over the count + 1 regions of the per-region mean square
+    rms = torch.sqrt(((applied - chain) ** 2).mean())
     adjoints = [chain[:, r].to(g_last_input.dtype) for r in range(count + 1)]
     return adjoints, float(rms.item())
 

@@ -10,7 +10,7 @@ from collections.abc import Sequence
 
 import torch
 
-from ..hip.interface import matrix_norms, suffix_scan_cotangents
+from ..hip.interface import matrix_norms, suffix_apply, suffix_scan_cotangents
 from ..hip.interface import suffix_scan_pullbacks as suffix_scan_jacobian_t
 
 
@@ -105,14 +105,12 @@ def propagate_state_adjoint_with_jacobian_scan(
         # The reference reaches its length check with an empty suffix list here.
         raise ValueError("suffix length mismatch.")
     if materialize_suffix:
-        suffix = compose_suffix_jacobian_t(state_jacobians_t)
-        if len(suffix) != count + 1:
+        suffix = suffix_scan_jacobian_t(_stack_for_chain(state_jacobians_t))
+        if suffix.shape[1] != count + 1:
             raise ValueError("suffix length mismatch.")
-        g_top_state = g_top_state.to(device=suffix[0].device, dtype=suffix[0].dtype)
-        g_states = [
-            apply_jacobian_t(suffix[region_index], g_top_state, out_dtype=g_top_state.dtype)
-            for region_index in range(count)
-        ]
+        g_top_state = g_top_state.to(device=suffix.device, dtype=suffix.dtype)
+        applied = suffix_apply(suffix, g_top_state)   # the K mat-vecs of the reference (and the identity) in one launch
+        g_states = [applied[:, region_index] for region_index in range(count)]
         g_states.append(g_top_state)
         return g_states
     stacked = _stack_for_chain(state_jacobians_t)

@@ -699,30 +699,48 @@ __global__ __launch_bounds__(512) void cotangent256_half_kernel(const Tin* __res
     }
 }
 
-// cot[b, r] = out[b, r] @ g[b] for every finished suffix product (r = K is the identity: cot[b, K] = g[b]): the
-// cotangents of the K-parallel scan, whose chunks have no common chain to carry them.  One workgroup per
-// (b, r), a wave per row at a time, lanes along k (16-byte loads), butterfly fold.  d a multiple of 4.
+// cot[b, r] = out[b, r] @ g[b] for M matrices per batch element: the cotangents of the K-parallel scan, whose
+// chunks have no common chain to carry them (M = K + 1; the identity tail gives cot[b, K] = g[b]), and the
+// entry point lbi_suffix_apply.  One workgroup per (b, r), a wave per row at a time, lanes along k (16-byte loads
+// when d is a multiple of 4), butterfly fold.
+template <bool VEC4>
 __global__ __launch_bounds__(256) void suffix_apply_kernel(const float* __restrict__ out, const float* __restrict__ g,
-                                                           float* __restrict__ cot, int K, int d) {
-    const int b = blockIdx.x / (K + 1);
+                                                           float* __restrict__ cot, int M, int d) {
+    const int b = blockIdx.x / M;
     const float* mat = out + (size_t)blockIdx.x * d * d;
     const float* g_b = g + (size_t)b * d;
     float* cot_r = cot + (size_t)blockIdx.x * d;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int row = wave; row < d; row += 4) {
         float acc = 0.0f;
-        for (int k = lane * 4; k < d; k += 256) {
-            const f32x4 a4 = *reinterpret_cast<const f32x4*>(mat + (size_t)row * d + k);
-            const f32x4 v4 = *reinterpret_cast<const f32x4*>(g_b + k);
-            acc = fmaf(a4[0], v4[0], acc);
-            acc = fmaf(a4[1], v4[1], acc);
-            acc = fmaf(a4[2], v4[2], acc);
-            acc = fmaf(a4[3], v4[3], acc);
+        if (VEC4) {
+            for (int k = lane * 4; k < d; k += 256) {
+                const f32x4 a4 = *reinterpret_cast<const f32x4*>(mat + (size_t)row * d + k);
+                const f32x4 v4 = *reinterpret_cast<const f32x4*>(g_b + k);
+                acc = fmaf(a4[0], v4[0], acc);
+                acc = fmaf(a4[1], v4[1], acc);
+                acc = fmaf(a4[2], v4[2], acc);
+                acc = fmaf(a4[3], v4[3], acc);
+            }
+        } else {
+            for (int k = lane; k < d; k += 64) acc = fmaf(mat[(size_t)row * d + k], g_b[k], acc);
         }
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
         if (lane == 0) cot_r[row] = acc;
     }
+}
+
+int launch_suffix_apply(const void* suffix, const void* g, void* cot, int64_t B, int64_t M, int d, hipStream_t stream) {
+    const dim3 grid((unsigned)(B * M));
+    if (d % 4 == 0)
+        hipLaunchKernelGGL(suffix_apply_kernel<true>, grid, dim3(256), 0, stream, static_cast<const float*>(suffix),
+                           static_cast<const float*>(g), static_cast<float*>(cot), (int)M, d);
+    else
+        hipLaunchKernelGGL(suffix_apply_kernel<false>, grid, dim3(256), 0, stream, static_cast<const float*>(suffix),
+                           static_cast<const float*>(g), static_cast<float*>(cot), (int)M, d);
+    LBI_HIP_CHECK(hipGetLastError());
+    return LBI_OK;
 }
 
 template <typename Tin, int D, int RT, int CB, bool COT, int MODE = 0>
@@ -785,11 +803,7 @@ int launch_chunked(const void* mats, void* out, const void* g, void* cot, int B,
                            : launch_mfma_cot<Tin, D, RT, CB, false, 1>(mats, out, nullptr, nullptr, B, K, stream, plan);
         if (rc) return rc;
     }
-    if (cot) {
-        hipLaunchKernelGGL(suffix_apply_kernel, dim3((unsigned)(B * (K + 1))), dim3(256), 0, stream,
-                           static_cast<const float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), K, D);
-        LBI_HIP_CHECK(hipGetLastError());
-    }
+    if (cot) return launch_suffix_apply(out, g, cot, B, K + 1, D, stream);
     return LBI_OK;
 }
 
@@ -1001,4 +1015,21 @@ extern "C" int lbi_suffix_cotangents(const void* mats, const void* g, void* out,
         case LBI_F16: return launch_cotangent<_Float16>(mats, g, out, (int)B, (int)K, (int)d, stream);
         default: return launch_cotangent<bf16_raw>(mats, g, out, (int)B, (int)K, (int)d, stream);
     }
+}
+
+extern "C" int lbi_suffix_apply(const void* suffix, const void* g, void* out, int64_t B, int64_t M, int64_t d,
+                                void* stream_v) {
+    using namespace lbi;
+    clear_error();
+    if (B < 0 || M < 0 || d < 0)
+        return fail(LBI_ERR_INVALID, "lbi_suffix_apply: negative size (B=%lld M=%lld d=%lld)", (long long)B,
+                    (long long)M, (long long)d);
+    if (d > 8192 || (double)B * (double)M > 2.0e9)
+        return fail(LBI_ERR_UNSUPPORTED, "lbi_suffix_apply: size out of range (B=%lld M=%lld d=%lld)", (long long)B,
+                    (long long)M, (long long)d);
+    if (B == 0 || M == 0 || d == 0) return LBI_OK;
+    if (!suffix || !g || !out) return fail(LBI_ERR_INVALID, "lbi_suffix_apply: null pointer");
+    if (d % 4 == 0 && (reinterpret_cast<uintptr_t>(suffix) % 16 || reinterpret_cast<uintptr_t>(g) % 16))
+        return fail(LBI_ERR_INVALID, "lbi_suffix_apply: suffix and g must be 16-byte aligned");
+    return launch_suffix_apply(suffix, g, out, B, M, (int)d, static_cast<hipStream_t>(stream_v));
 }

@@ -118,6 +118,29 @@ def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor) ->
     return out, cot
 
 
+def suffix_apply(suffix: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """``out[b, r] = suffix[b, r] @ g[b]`` for every matrix of ``suffix [B, M, d, d]`` (fp32, as the scan returns
+    it; other float types are converted) in one launch: the mat-vecs of reference backward/suffix_scan.py:49-53."""
+    if not isinstance(suffix, torch.Tensor) or suffix.dim() != 4 or suffix.shape[-1] != suffix.shape[-2]:
+        raise ValueError("suffix must have shape [B, M, R, R]")
+    bsz, count, rank, _ = suffix.shape
+    if g.dim() != 2 or g.shape[0] != bsz or g.shape[1] != rank:
+        raise ValueError("g must have shape [B, R]")
+    if not suffix.is_cuda:
+        raise RuntimeError("suffix must be a CUDA tensor (this build has no CPU execution path)")
+    suffix = suffix.to(torch.float32).contiguous()
+    g32 = g.to(device=suffix.device, dtype=torch.float32).contiguous()
+    out = torch.empty((bsz, count, rank), device=suffix.device, dtype=torch.float32)
+    if out.numel() == 0:
+        return out
+    lib = _lib.load()
+    with torch.cuda.device(suffix.device):
+        status = lib.lbi_suffix_apply(suffix.data_ptr(), g32.data_ptr(), out.data_ptr(), bsz, count, rank,
+                                      _lib.current_stream_ptr(suffix.device))
+    _lib.check(status, "lbi_suffix_apply")
+    return out
+
+
 def matrix_norms(mats: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """``(spectral, frobenius)`` norms, fp32, of every square matrix of ``mats [..., d, d]``.
 
@@ -153,4 +176,5 @@ def matrix_norms(mats: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return spectral, frobenius
 
 
-__all__ = ["matrix_norms", "suffix_scan_pullbacks", "suffix_scan_cotangents", "suffix_scan_pullbacks_and_cotangents"]
+__all__ = ["matrix_norms", "suffix_apply", "suffix_scan_pullbacks", "suffix_scan_cotangents",
+           "suffix_scan_pullbacks_and_cotangents"]

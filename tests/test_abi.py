@@ -48,6 +48,13 @@ def test_argument_validation_needs_no_gpu():
     assert lib.lbi_suffix_scan(None, None, 0, 2, 4, _lib.LBI_F32, _lib.LBI_F32, None) == 0
     assert lib.lbi_last_error() == b""
     assert lib.lbi_suffix_cotangents(None, None, None, 1, 2, 4, _lib.LBI_F32, None) == -1
+    assert lib.lbi_suffix_apply(None, None, None, 1, 2, 4, None) == -1
+    assert b"null" in lib.lbi_last_error()
+    assert lib.lbi_suffix_apply(None, None, None, -1, 2, 4, None) == -1
+    assert lib.lbi_suffix_apply(None, None, None, 0, 2, 4, None) == 0
+    odd = ctypes.c_void_p(260)  # not 16-byte aligned
+    assert lib.lbi_suffix_apply(odd, odd, odd, 1, 2, 4, None) == -1
+    assert b"aligned" in lib.lbi_last_error()
 
 
 def test_region_and_norm_entry_points_validate_on_the_host():

@@ -296,6 +296,23 @@ def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, device):
     assert res.returncode == 0, res.stdout + res.stderr
 
 
+@pytest.mark.parametrize("shape", [(1, 1, 1), (2, 4, 5), (3, 6, 16), (2, 9, 64), (1, 3, 100), (2, 5, 256), (1, 2, 300)])
+def test_suffix_apply_matches_einsum(shape, device):
+    """``lbi_suffix_apply``: every matrix of a stack applied to its batch element's vector, in fp64 on the CPU."""
+    from latent_bounded_interfaces_amd.hip.interface import suffix_apply
+
+    bsz, count, rank = shape
+    gen = torch.Generator().manual_seed(rank)
+    suffix = torch.randn(bsz, count, rank, rank, generator=gen)
+    g = torch.randn(bsz, rank, generator=gen)
+    got = suffix_apply(suffix.to(device), g.to(device)).cpu()
+    want = torch.einsum("bkij,bj->bki", suffix.double(), g.double())
+    assert got.shape == (bsz, count, rank) and got.dtype == torch.float32
+    assert torch.allclose(got.double(), want, atol=1e-5 * float(want.abs().max()), rtol=1e-5)
+    with pytest.raises(ValueError):
+        suffix_apply(suffix.to(device), g[:, :-1].to(device)) if rank > 1 else suffix_apply(suffix[0].to(device), g.to(device))
+
+
 def test_backward_module_contract(device):
     """Counterpart functions of reference backward/suffix_scan.py keep its edge cases."""
     from latent_bounded_interfaces_amd.backward import suffix_scan as bs
