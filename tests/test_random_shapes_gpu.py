@@ -82,3 +82,36 @@ def test_16bit_cotangent_chain_random_lengths(device):
         truth = oscan.suffix_cotangents_sequential(mats.double(), g.double())
         scale = truth.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
         assert float(((out.double() - truth).abs() / scale).max()) <= 1e-5, (case, bsz, count, dtype)
+
+
+def test_suffix_scan_random_shapes(device):
+    """The scan entries over random batch sizes, chain lengths and widths (matrix-core widths, padded widths,
+    scalar widths; chains short and long enough for the K-parallel form; every storage type): matrices against the
+    fp64 sequential product at the fp32 bar, cotangents at the bars of their two forms, fused == separate."""
+    from latent_bounded_interfaces_amd.hip.interface import (suffix_scan_cotangents, suffix_scan_pullbacks,
+                                                             suffix_scan_pullbacks_and_cotangents)
+
+    rng = random.Random(3)
+    for case in range(28):
+        rank = rng.choice([32, 64, 128, 256, 256, 64, rng.randint(1, 40), rng.randint(41, 200)])
+        count = rng.choice([0, 1, 2, rng.randint(3, 11), rng.randint(12, 40), rng.randint(41, 90)])
+        bsz = rng.choice([1, 1, 2, 3, rng.randint(4, 9), rng.randint(10, 20)])
+        if rank > 128:
+            count, bsz = min(count, 48), min(bsz, 6)
+        dtype = rng.choice([torch.float32, torch.float32, torch.bfloat16, torch.float16])
+        kind = rng.choice(["randn", "near_identity"])
+        mats, g = oscan.make_scan_inputs(bsz, count, rank, kind=kind, seed=300 + case)
+        mats = mats.to(dtype)
+        tag = (case, bsz, count, rank, dtype, kind)
+        out, cot = suffix_scan_pullbacks_and_cotangents(mats.to(device), g.to(device))
+        assert torch.equal(out, suffix_scan_pullbacks(mats.to(device))), tag
+        truth = oscan.suffix_scan_sequential(mats.float(), dtype=torch.float64)
+        err = (out.cpu().double() - truth).abs().flatten(2).amax(2) / truth.abs().flatten(2).amax(2).clamp_min(1e-30)
+        assert float(err.max()) <= 1e-5, tag
+        assert torch.equal(out[:, count].cpu(), torch.eye(rank).expand(bsz, rank, rank)), tag
+        want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+        scale = want.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+        # the fused entry's cotangents are the chain, or in its K-parallel form the products applied to g (3e-5)
+        assert float(((cot.cpu().double() - want).abs() / scale).max()) <= 3e-5, tag
+        chain = suffix_scan_cotangents(mats.to(device), g.to(device)).cpu()
+        assert float(((chain.double() - want).abs() / scale).max()) <= 1e-5, tag
