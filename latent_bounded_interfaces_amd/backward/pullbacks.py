@@ -77,14 +77,17 @@ class StructuredInterfacePullbackProvider:
             return first if flags[0] else g_region_output
         return first if bool(torch.equal(first, g_region_output)) else g_region_output
 
-    def region_state_jacobian_t(self, *, model: Any, region_cache: Any, out: torch.Tensor | None = None) -> torch.Tensor:
-        """``Jt`` of one region, ``[B, d, d]``; written into ``out`` (any strides) when given."""
+    def region_state_jacobian_t(self, *, model: Any, region_cache: Any, out: torch.Tensor | None = None,
+                                dtype: torch.dtype | None = None) -> torch.Tensor:
+        """``Jt`` of one region, ``[B, d, d]``; written into ``out`` (any strides) when given.  ``dtype``: dtype of
+        the cotangent basis and of the result (default: that of ``out``, else of the region's input state)."""
         state_in = region_cache.state_in
         if state_in.dim() != 2:
             raise ValueError("interface state inputs must be [B, R].")
         bsz, rank = state_in.shape
         chunk = self.basis_chunk or rank
-        eye = torch.eye(rank, device=state_in.device, dtype=state_in.dtype)
+        dtype = dtype or (out.dtype if out is not None else state_in.dtype)
+        eye = torch.eye(rank, device=state_in.device, dtype=dtype)
         cols: list[torch.Tensor] = []
         with torch.no_grad():
             for start in range(0, rank, chunk):
@@ -103,7 +106,7 @@ class StructuredInterfacePullbackProvider:
                     cols.append(total.transpose(1, 2))                    # [B, d_in, P]
         if out is not None:
             return out
-        return torch.cat(cols, dim=-1).to(device=state_in.device, dtype=state_in.dtype).contiguous()
+        return torch.cat(cols, dim=-1).to(device=state_in.device, dtype=dtype).contiguous()
 
     def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
         """One ``[B, d, d]`` tensor per region.  The first K - 1 of them are slices of ONE dense ``[B, K-1, d, d]``
@@ -118,10 +121,14 @@ class StructuredInterfacePullbackProvider:
             return [self.region_state_jacobian_t(model=model, region_cache=rc) for rc in region_caches]
         state = region_caches[0].state_in
         bsz, rank = state.shape
-        inner = torch.empty((bsz, count - 1, rank, rank), device=state.device, dtype=state.dtype)
+        # one dtype for all regions: a forward under autocast can leave the first state 16-bit and the others fp32
+        dtype = state.dtype
+        for rc in region_caches[1:]:
+            dtype = torch.promote_types(dtype, rc.state_in.dtype)
+        inner = torch.empty((bsz, count - 1, rank, rank), device=state.device, dtype=dtype)
         result = [self.region_state_jacobian_t(model=model, region_cache=rc, out=inner[:, r])
                   for r, rc in enumerate(region_caches[:-1])]
-        result.append(self.region_state_jacobian_t(model=model, region_cache=region_caches[-1]))
+        result.append(self.region_state_jacobian_t(model=model, region_cache=region_caches[-1], dtype=dtype))
         return result
 
 

@@ -261,6 +261,9 @@ def _apply_transposed(g: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``g @ weight`` for ``weight [out, in]``: the pullback of ``y = x weight^T``.  For tall ``g`` it is issued as
     the library's ``A B^T`` form on a transposed copy of the (small) weight, which is its faster path for these
     products; for few rows (the single direction of a parameter VJP) the copy is not worth it."""
+    if weight.dtype != g.dtype:
+        # a forward run under autocast multiplied by the weight cast to the compute dtype; so does its pullback
+        weight = weight.to(g.dtype)
     if g.numel() // g.shape[-1] < _TRANSPOSED_COPY_MIN_ROWS:
         return torch.matmul(g, weight)
     return torch.nn.functional.linear(g, weight.t().contiguous())
@@ -334,8 +337,11 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
     parameter gradients of the block are formed on the way, each from the cotangent at the
     output of its module and the cached input of that module."""
     attn, mlp = block.attn, block.mlp
-    wdtype = mlp.fc2.weight.dtype
     a_cache, m_cache = layer_cache.attention, layer_cache.mlp
+    # Branch cotangents live in the dtype the forward's matrix products ran in, which is what the cached
+    # attention operands have: the weights' own dtype, or the autocast dtype of a mixed-precision forward
+    # (fp32 master weights, 16-bit products; reference train/runners.py:361), whose weights are cast per use.
+    wdtype = a_cache.q_rope.dtype
     if g_hidden is None:
         g_hidden = g_residual.to(wdtype)
 
@@ -380,7 +386,8 @@ def _layer_input_pullback(block: Any, layer_cache: Any, g_hidden: torch.Tensor |
             if param_grads is not None:
                 # the cache keeps the projection after the convolution only: redo the projection
                 bias = getattr(attn.in_proj, "bias", None)
-                x_pre = torch.nn.functional.linear(a_cache.norm_output, attn.in_proj.weight, bias)
+                x_pre = torch.nn.functional.linear(a_cache.norm_output.to(wdtype), attn.in_proj.weight.to(wdtype),
+                                                   None if bias is None else bias.to(wdtype))
                 _conv_grads(param_grads, attn.conv1d, g_qkv, x_pre)
                 del x_pre
             g_qkv = causal_conv1d_pullback(g_qkv, attn.conv1d.weight)

@@ -80,11 +80,15 @@ class OracleVectorInterface(nn.Module):
         return [self.update_scale]
 
     @staticmethod
-    def _vjp_rows(fn, x, g_out):
-        """g_out [B, P, O] pulled back through fn at x [B, I] -> [B, P, I]."""
+    def _vjp_rows(fn, x, g_out, dtype=None):
+        """g_out [B, P, O] pulled back through fn at x [B, I] -> [B, P, I].  ``dtype``: the dtype fn computes in
+        (its parameters'); a forward run under autocast leaves some interface activations and states in the
+        autocast dtype, while the pullback runs outside autocast."""
         bsz, basis = g_out.shape[:2]
+        dtype = dtype or g_out.dtype
         with torch.enable_grad():
-            x_rep = x.detach().unsqueeze(1).expand(bsz, basis, x.shape[-1]).reshape(bsz * basis, -1).requires_grad_(True)
+            x_rep = (x.detach().to(dtype).unsqueeze(1).expand(bsz, basis, x.shape[-1]).reshape(bsz * basis, -1)
+                     .requires_grad_(True))
             y = fn(x_rep)
             (g_in,) = torch.autograd.grad(y, x_rep, grad_outputs=g_out.reshape_as(y).to(y.dtype))
         return g_in.reshape(bsz, basis, -1).to(g_out.dtype)
@@ -94,7 +98,8 @@ class OracleVectorInterface(nn.Module):
             raise ValueError("state_out_cotangent_basis must have shape [B, P, R].")
         r = region_cache.region_index
         diag = region_cache.interface_step.diagnostics
-        g_pre = self._vjp_rows(self.norms[r], diag["pre_norm_state"], state_out_cotangent_basis)
+        g_pre = self._vjp_rows(self.norms[r], diag["pre_norm_state"], state_out_cotangent_basis,
+                              dtype=self.norms[r].weight.dtype)
         g_delta = g_pre * diag["update_scale"].to(g_pre.dtype)
         g_pooled = self._vjp_rows(lambda t: self._run(self.encoders[r], t), diag["pooled_features"], g_delta)
         seq_len = region_cache.region_output.shape[1]

@@ -287,3 +287,57 @@ def test_16bit_step_at_real_head_geometry_reproduces_dense_gradients(dtype, devi
     got_jt = engine.pullback_provider.materialize_state_jacobian_t(model=model, cache=cache)
     for a, b in zip(got_jt, want_jt):
         assert float((a.float() - b).abs().max()) <= 2e-2 * float(b.abs().max())
+
+
+def test_step_on_an_autocast_forward_with_fp32_master_weights(device):
+    """The reference's training loop keeps fp32 weights and runs the forward under ``autocast(bfloat16)``
+    (train/runners.py:299, :361): the cache then holds 16-bit attention / MLP activations beside an fp32 residual
+    stream and fp32 weights.  The structured provider follows the forward's compute dtype (weights cast per use);
+    state Jacobians against the autograd graph of that same forward, step gradients against its dense backward."""
+    from latent_bounded_interfaces_amd.backward import ScanADEngine
+
+    model = _model(device, dim=128, n_heads=2, n_kv_heads=1, hidden=256, layers=4, layers_per_region=2,
+                   interface_width=16, interface_hidden=24, seed=41)
+    gen = torch.Generator().manual_seed(10)
+    ids = torch.randint(0, 61, (2, 192), generator=gen).to(device)
+    targets = torch.randint(0, 61, (2, 192), generator=gen).to(device)
+
+    def forward():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits, cache = model.forward_with_cache(ids)
+        return olbi.token_loss(logits, targets), cache
+
+    model.zero_grad(set_to_none=True)
+    loss, cache = forward()
+    loss.backward()
+    dense = {n: (None if p.grad is None else p.grad.detach().clone()) for n, p in model.named_parameters()}
+    model.zero_grad(set_to_none=True)
+
+    loss, cache = forward()
+    layer0 = cache["region_caches"][0].backend_cache.layer_caches[0]
+    assert layer0.attention.q_rope.dtype == torch.bfloat16 and layer0.mlp.norm_input.dtype == torch.float32
+    assert next(model.region_backend.parameters()).dtype == torch.float32
+    engine = ScanADEngine(state_jacobian_mode="structured", state_jacobian_basis_chunk=0)
+    want_jt = olbi.GraphInterfacePullbackProvider().materialize_state_jacobian_t(model=model, cache=cache)
+    got_jt = engine.pullback_provider.materialize_state_jacobian_t(model=model, cache=cache)
+    for a, b in zip(got_jt, want_jt):
+        # the graph provider returns region 0 in the 16-bit dtype of the first state; here all regions share fp32
+        assert a.dtype == torch.float32
+        assert float((a - b.float()).abs().max()) <= 2e-2 * float(b.abs().max()), float((a - b.float()).abs().max())
+    result = engine.backward(model=model, loss=loss, cache=cache)
+    assert result.diagnostics["interface_scan_rms"] < 5e-5
+    for name, want in dense.items():
+        got = result.grad_map[name]
+        assert (got is None) == (want is None), name
+        if want is None:
+            continue
+        assert got.dtype == want.dtype == torch.float32
+        rel = float((got - want).norm() / want.norm().clamp_min(1e-12))
+        assert rel <= 5e-2, (name, rel)
+        assert torch.allclose(got, want, atol=5e-2, rtol=5e-2), name
+    # parameter_vjp of a region on the same cache: fp32 gradients for fp32 parameters
+    cot = torch.randn(2, 192, 128, device=device)
+    rc = cache["region_caches"][1].backend_cache
+    grads = model.region_backend.lowering.parameter_vjp(backend=model.region_backend, cache=rc, output_cotangent=cot)
+    params = dict(model.region_backend.named_parameters())
+    assert grads and all(g.dtype == params[n].dtype and g.shape == params[n].shape for n, g in grads.items())
