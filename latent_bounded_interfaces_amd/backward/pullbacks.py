@@ -108,16 +108,26 @@ class StructuredInterfacePullbackProvider:
             return out
         return torch.cat(cols, dim=-1).to(device=state_in.device, dtype=dtype).contiguous()
 
-    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
+    #: ``materialize_state_jacobian_t`` takes ``skip_last=True``: the scan backward step asks for that when nothing
+    #: reads the last region's Jacobian (one region pullback less per step)
+    can_skip_last_region = True
+
+    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any],
+                                     skip_last: bool = False) -> list[torch.Tensor]:
         """One ``[B, d, d]`` tensor per region.  The first K - 1 of them are slices of ONE dense ``[B, K-1, d, d]``
         buffer, in order: the scan backward step composes exactly those (the last region's output state never
         reaches the loss, reference backward/suffix_scan.py:71), and ``backward.suffix_scan`` hands such a list to
-        the kernels as it lies, without the stacking copy (reference backward/suffix_scan.py:17)."""
+        the kernels as it lies, without the stacking copy (reference backward/suffix_scan.py:17).
+
+        ``skip_last=True`` leaves the last region's Jacobian out (``None`` in its place): the reference builds it
+        and drops it (backward/scan.py:44, backward/suffix_scan.py:71-74); only the Jacobian statistics read it."""
         region_caches = cache["region_caches"]
         count = len(region_caches)
         if count != model.num_regions:
             raise ValueError("cache has invalid region_caches length.")
         if count < 2:
+            if skip_last:
+                return [None for _ in region_caches]
             return [self.region_state_jacobian_t(model=model, region_cache=rc) for rc in region_caches]
         state = region_caches[0].state_in
         bsz, rank = state.shape
@@ -128,7 +138,8 @@ class StructuredInterfacePullbackProvider:
         inner = torch.empty((bsz, count - 1, rank, rank), device=state.device, dtype=dtype)
         result = [self.region_state_jacobian_t(model=model, region_cache=rc, out=inner[:, r])
                   for r, rc in enumerate(region_caches[:-1])]
-        result.append(self.region_state_jacobian_t(model=model, region_cache=region_caches[-1], dtype=dtype))
+        result.append(None if skip_last else
+                      self.region_state_jacobian_t(model=model, region_cache=region_caches[-1], dtype=dtype))
         return result
 
 

@@ -8,6 +8,9 @@ keys, same order of calls into the local-VJP provider, same edge cases (no regio
 * the state adjoints and the suffix matrices come from ONE launch
   (``lbi_suffix_scan_with_cotangents``): the adjoints are the chain ``g_r = Jt_r g_{r+1}`` carried
   beside the matrix products;
+* the last region's state Jacobian, which the reference builds and then drops (its output state never reaches the
+  loss), is not built when the provider can leave it out and the Jacobian statistics are off: one region pullback
+  less per step;
 * ``interface_scan_rms`` (logged by the reference's training loop as ``scan_align``) is reported
   on every step as the reference does (:63-72), from the two independent results that launch
   yields: the chain, and the suffix matrices applied to the last cotangent (one more launch
@@ -73,7 +76,12 @@ def lbi_scan_backward_step(
         g_state_inputs = [local_vjp_provider.state_adjoint_from_loss(loss=ce_loss, state=states[0])]
     else:
         g_last_input = local_vjp_provider.state_adjoint_from_loss(loss=ce_loss, state=states[-2])
-        state_jacobians_t = pullback_provider.materialize_state_jacobian_t(model=model, cache=cache)
+        # The last region's Jacobian is read by the statistics only (the reference builds it every step and drops
+        # it, backward/suffix_scan.py:71-74): a provider that can leave it out is asked to.
+        if not compute_interface_jacobian_stats and getattr(pullback_provider, "can_skip_last_region", False):
+            state_jacobians_t = pullback_provider.materialize_state_jacobian_t(model=model, cache=cache, skip_last=True)
+        else:
+            state_jacobians_t = pullback_provider.materialize_state_jacobian_t(model=model, cache=cache)
         g_last_input = g_last_input.to(device=state_jacobians_t[0].device, dtype=state_jacobians_t[0].dtype)
         if compute_interface_jacobian_stats:
             interface_jacobian_stats = interface_state_jacobian_t_stats(

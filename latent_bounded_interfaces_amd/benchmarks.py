@@ -340,10 +340,11 @@ def measure_lbi_step(*, regions=6, layers_per_region=2, dim=768, n_heads=12, hea
                      batch=8, seq_len=1024, interface_width=64, dtype=torch.bfloat16, warmup=1, iters=3,
                      device="cuda") -> dict:
     """Device work of one LBI scan backward step at the end-to-end configuration (12 layers in 6
-    regions of 2, interface width 64): per region the state-Jacobian build (region input pullback
-    for 64 directions) and the parameter VJP, then the interface suffix scan (cotangent chain over
-    the 5 inner Jacobians).  The region-output cotangents are constant over positions (mean-pooling
-    interface).  The forward caches are synthetic and shared by the six regions
+    regions of 2, interface width 64): the state-Jacobian build (region input pullback for 64
+    directions) of every region but the last, whose Jacobian the step leaves out (the reference
+    builds all six and drops the last), the parameter VJP of every region, and the interface suffix scan
+    (cotangent chain over the 5 inner Jacobians).  The region-output cotangents are constant over positions
+    (mean-pooling interface).  The forward caches are synthetic and shared by the six regions
     (same shapes); the interface's own small MLP pullbacks and the readout/canvas VJPs are not part
     of this library and are left out."""
     from .backends import HipTransformerLowering
@@ -364,7 +365,7 @@ def measure_lbi_step(*, regions=6, layers_per_region=2, dim=768, n_heads=12, hea
     parts = {}
 
     def pullbacks():
-        for _ in range(regions):
+        for _ in range(regions - 1):
             lowering.input_pullback_basis(backend=backend, cache=cache, output_cotangent_basis=basis)
 
     def vjps():
@@ -384,6 +385,7 @@ def measure_lbi_step(*, regions=6, layers_per_region=2, dim=768, n_heads=12, hea
         median_ms, best_ms, mean_ms, peak = time_call(fn, warmup=warmup, iters=iters)
         parts[name] = {"median_ms": median_ms, "best_ms": best_ms, "peak_memory_bytes": peak}
     return {
+        "state_jacobians_built": regions - 1,
         "workload": f"LBI scan backward step, device work: {regions} regions x {layers_per_region} layers, d_model {dim}, "
                     f"{n_heads} heads x {head_dim}, hidden {hidden}, interface width {interface_width}, B={batch} "
                     f"T={seq_len}, {str(dtype).replace('torch.', '')}, synthetic caches",

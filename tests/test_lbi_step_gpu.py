@@ -341,3 +341,61 @@ def test_step_on_an_autocast_forward_with_fp32_master_weights(device):
     grads = model.region_backend.lowering.parameter_vjp(backend=model.region_backend, cache=rc, output_cotangent=cot)
     params = dict(model.region_backend.named_parameters())
     assert grads and all(g.dtype == params[n].dtype and g.shape == params[n].shape for n, g in grads.items())
+
+
+def test_step_leaves_out_the_last_regions_jacobian_unless_statistics_read_it(device):
+    """The last region's state Jacobian never enters the adjoints (reference backward/suffix_scan.py:71-74).  The
+    step asks the structured provider to leave it out: one region pullback less, the same gradients bit for bit as
+    with a provider that builds it; with the Jacobian statistics on it is built, since they report its norms."""
+    from latent_bounded_interfaces_amd.backward import StructuredInterfacePullbackProvider, lbi_scan_backward_step
+
+    model = _model(device)
+    gen = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, 61, (2, 10), generator=gen).to(device)
+    targets = torch.randint(0, 61, (2, 10), generator=gen).to(device)
+
+    class BuildsAll:
+        """The same provider without the option."""
+        name = "structured"
+
+        def __init__(self):
+            self.inner = StructuredInterfacePullbackProvider()
+
+        def materialize_state_jacobian_t(self, *, model, cache):
+            return self.inner.materialize_state_jacobian_t(model=model, cache=cache)
+
+    calls = []
+    inner = model.region_backend.input_pullback_basis
+
+    def spy(*, cache, output_cotangent_basis):
+        calls.append(cache.region_index)
+        return inner(cache=cache, output_cotangent_basis=output_cotangent_basis)
+
+    def step(provider, **kw):
+        logits, cache = model.forward_with_cache(ids)
+        loss = olbi.token_loss(logits, targets)
+        calls.clear()
+        model.region_backend.input_pullback_basis = spy
+        try:
+            result = lbi_scan_backward_step(model, ce_loss=loss, cache=cache, pullback_provider=provider, **kw)
+        finally:
+            del model.region_backend.input_pullback_basis
+        return result, list(calls), cache
+
+    got, got_calls, cache = step(StructuredInterfacePullbackProvider())
+    want, want_calls, _ = step(BuildsAll())
+    assert got_calls == [0, 1] and want_calls == [0, 1, 2]
+    assert got.interface_scan_rms == want.interface_scan_rms
+    assert set(got.grad_map) == set(want.grad_map)
+    for name, value in want.grad_map.items():
+        assert (got.grad_map[name] is None) == (value is None), name
+        if value is not None:
+            assert torch.equal(got.grad_map[name], value), name
+    with_stats, stats_calls, _ = step(StructuredInterfacePullbackProvider(), compute_interface_jacobian_stats=True)
+    assert stats_calls == [0, 1, 2] and with_stats.interface_jacobian_stats is not None
+    # the provider's own contract
+    provider = StructuredInterfacePullbackProvider()
+    full = provider.materialize_state_jacobian_t(model=model, cache=cache)
+    short = provider.materialize_state_jacobian_t(model=model, cache=cache, skip_last=True)
+    assert len(short) == len(full) == 3 and short[-1] is None
+    assert all(torch.equal(a, b) for a, b in zip(short[:-1], full[:-1]))
