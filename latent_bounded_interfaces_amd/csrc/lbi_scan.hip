@@ -768,14 +768,18 @@ int launch_mfma(const void* mats, void* out, const void* g, void* cot, int B, in
 
 // Chunking of the K-parallel scan: C chunks of L matrices.  The dependent depth is 2L + C - 3 steps, least at
 // L ~ sqrt(K / 2).  The chunked form does twice the products, which is free only while the plain form (B * nb
-// workgroups) leaves at least half of the 256 CUs idle; C is capped so that the widest phase stays within two
-// workgroups per CU.  Measured at K = 128 (plain -> chunked, ms): d = 256: B = 1: 2.36 -> 0.28, 8: 2.04 -> 0.58,
-// 16: 2.05 -> 1.05, 32: 2.07 -> 1.8-2.1 (not taken); d = 128: B = 16: 0.35 -> 0.21, 48: 0.43 -> 0.57 (not taken).
+// workgroups) leaves at least half of the 256 CUs idle; C is capped so that the widest phase stays within one
+// workgroup per CU, or within two where one would leave fewer than five chunks.  Measured at K = 128 (plain ->
+// chunked, ms per call): d = 256: B = 1: 2.36 -> 0.29, 4: 2.37 -> 0.37, 8: 2.04 -> 0.59, 16: 2.05 -> 1.14,
+// 32: 2.07 -> 2.3 (not taken); d = 128: B = 16: 0.35 -> 0.19, 48: 0.43 -> 0.57 (not taken).
 // Returns false when the plain chain is at least as good.  LBI_SCAN_CHUNK=0 forces the plain chain, n >= 2 chunks of n.
 inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
     static const int forced = std::getenv("LBI_SCAN_CHUNK") ? std::atoi(std::getenv("LBI_SCAN_CHUNK")) : -1;
     if (forced == 0) return false;
-    const int cmax = 512 / (B * nb) + 1;
+    // chunks side by side: one workgroup per CU while that still leaves five or more of them (a step of two
+    // workgroups sharing a CU takes 1.7x as long), else two per CU
+    const int one_per_cu = 256 / (B * nb) + 1;
+    const int cmax = one_per_cu >= 5 ? one_per_cu : 512 / (B * nb) + 1;
     if (K < 12 || ((B * nb > 128 || cmax < 4) && forced <= 0)) return false;
     int L = 2;
     while (2 * (L + 1) * (L + 1) <= K) ++L;  // floor(sqrt(K / 2))
