@@ -63,10 +63,15 @@ struct ScanPlan {
     int phase;  // 0: whole chain; 1, 2, 3: see above
     int L;      // matrices per chunk (>= 2)
     int C;      // chunks (>= 3)
+    // One level of the log-depth form of phase 2 (MODE 3): element c = 1 .. C-2 lives in slot out[cL + rd], the
+    // last element is out[(C-1)L]; the level writes elem[c] @ elem[c + off] (or elem[c] itself where c + off is
+    // past the last element) to out[cL + wr].
+    int off, rd, wr;
 };
 
 // MODE 0: phase 0 only; every switch below is a compile-time constant, which keeps the whole-chain kernel at its
 // register count.  MODE 1: phases 1 and 3 (switches at run time, unit strides).  MODE 2: phase 2 (strided).
+// MODE 3: one level of phase 2 in log-depth form (one product per workgroup, all chunks side by side).
 template <typename Tin, int D, int RT, int CB, bool COT, int MODE>
 __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     const Tin* __restrict__ mats, float* __restrict__ out, const float* __restrict__ g,
@@ -86,7 +91,7 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     // A launch covers E = B * (segments per batch element) chains.  With at least 8 of them the workgroups are
     // dealt round-robin to the 8 XCDs so that all column blocks of one chain get ids that are equal mod 8 and
     // share one L2; smaller launches are sized exactly.
-    const int nseg = MODE == 1 ? plan.C - 1 : 1;
+    const int nseg = MODE == 1 ? plan.C - 1 : MODE == 3 ? plan.C - 2 : 1;
     const int E = B * nseg;
     const int id = blockIdx.x;
     int e, c0;
@@ -145,6 +150,26 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
             r_lo = c == 0 ? 0 : c * plan.L + 1;   // out[cL] is a phase 2 result already
             cot_init = c < plan.C - 2;            // out[(C-1)L] @ g is the last chunk's own chain value
         }
+    } else if constexpr (MODE == 3) {
+        const int c = seg + 1;
+        const float* left = out_b + ((size_t)c * plan.L + plan.rd) * DD;
+        float* dst = out_b + ((size_t)c * plan.L + plan.wr) * DD;
+        const int partner = c + plan.off;
+        if (partner > plan.C - 1) {
+            // nothing to the right at this distance: the element is complete, it moves to the level's output slot
+            for (int idx = threadIdx.x; idx < D * CB / 4; idx += NT) {
+                const int row = idx / (CB / 4), q = idx % (CB / 4);
+                *reinterpret_cast<f32x4*>(dst + (size_t)row * D + c0 + 4 * q) =
+                    *reinterpret_cast<const f32x4*>(left + (size_t)row * D + c0 + 4 * q);
+            }
+            return;
+        }
+        a_base = reinterpret_cast<const Tin*>(left);
+        o_base = dst;
+        init_s = partner == plan.C - 1 ? out_b + (size_t)(plan.C - 1) * plan.L * DD
+                                       : out_b + ((size_t)partner * plan.L + plan.rd) * DD;
+        r_top = 0;
+        cot_on = false;
     } else {
         // step j multiplies the total parked in out[(j+1)L + 1] and stores out[(j+1)L]
         a_base = reinterpret_cast<const Tin*>(out_b + (size_t)(plan.L + 1) * DD);
@@ -163,6 +188,27 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     {
         float* o_last = out_b + (size_t)(K - 1) * DD;
         float* o_eye = out_b + (size_t)K * DD;
+        if (MODE != 0) {
+            // the chunk phases are short chains: four elements per load, all loads of a thread in flight
+            constexpr int Q = CB / 4;
+            static_assert((D * Q) % NT == 0, "start-state fill");
+#pragma unroll
+            for (int u = 0; u < D * Q / NT; ++u) {
+                const int idx = tid + u * NT;
+                const int row = idx / Q, q = idx % Q;
+                const size_t off = (size_t)row * D + c0 + 4 * q;
+                const f32x4 v4 = from_a ? load4(init_a + off) : load4(init_s + off);
+                if (write_tail) {
+                    f32x4 eye = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) eye[t] = (row == c0 + 4 * q + t) ? 1.0f : 0.0f;
+                    *reinterpret_cast<f32x4*>(o_last + off) = v4;
+                    *reinterpret_cast<f32x4*>(o_eye + off) = eye;
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) lds[(4 * q + t) * PITCH + row] = v4[t];
+            }
+        } else {
         for (int idx = tid; idx < D * CB; idx += NT) {
             const int row = idx / CB;
             const int col = idx % CB;
@@ -172,6 +218,7 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 o_eye[row * D + c0 + col] = (row == c0 + col) ? 1.0f : 0.0f;
             }
             lds[col * PITCH + row] = val;
+        }
         }
         if (COT) {
             // first vector of the chain: (start state) @ g, one row per thread, once per kernel
@@ -745,14 +792,14 @@ int launch_suffix_apply(const void* suffix, const void* g, void* cot, int64_t B,
 
 template <typename Tin, int D, int RT, int CB, bool COT, int MODE = 0>
 int launch_mfma_cot(const void* mats, void* out, const void* g, void* cot, int B, int K, hipStream_t stream,
-                    ScanPlan plan = ScanPlan{0, 0, 0}) {
+                    ScanPlan plan = ScanPlan{0, 0, 0, 0, 0, 0}) {
     constexpr int NW = D / RT;
     constexpr int NB = D / CB;
     constexpr size_t lds_bytes = ((size_t)2 * CB * (D + 4) + (COT ? 2 * D : 0)) * sizeof(float);
     auto kern = scan_mfma_kernel<Tin, D, RT, CB, COT, MODE>;
     if (int rc = ensure_dynamic_lds<&scan_mfma_kernel<Tin, D, RT, CB, COT, MODE>>(lds_bytes)) return rc;
     // chains in this launch (the kernel derives the same number from the plan)
-    const int chains = B * (MODE == 1 ? plan.C - 1 : 1);
+    const int chains = B * (MODE == 1 ? plan.C - 1 : MODE == 3 ? plan.C - 2 : 1);
     const dim3 grid(chains >= 8 ? ((chains + 7) / 8) * 8 * NB : chains * NB);
     hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds_bytes, stream, static_cast<const Tin*>(mats),
                        static_cast<float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), B, K, plan);
@@ -800,11 +847,31 @@ inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
 template <typename Tin, int D, int RT, int CB>
 int launch_chunked(const void* mats, void* out, const void* g, void* cot, int B, int K, ScanPlan plan,
                    hipStream_t stream) {
+    // Phase 2 as a chain takes C - 2 dependent steps on B * D / CB workgroups.  With many chunks it runs in log
+    // depth instead: level l multiplies every element by the one 2^l places to its right, all chunks side by
+    // side, ceil(log2(C - 1)) launches of one step each.  The levels alternate between the two slots of a chunk
+    // that phase 3 rewrites anyway (out[cL + 1], where phase 1 parked the total, and out[cL + 2]: L >= 3) and the
+    // last one writes out[cL]; no slot is read and written in the same launch.
+    int levels = 0;
+    while ((1 << levels) < plan.C - 1) ++levels;
+    static const bool no_log = std::getenv("LBI_SCAN_TOTALS_CHAIN") && std::atoi(std::getenv("LBI_SCAN_TOTALS_CHAIN"));
+    const bool log_depth = !no_log && plan.L >= 3 && 2 * levels <= plan.C - 2;
     for (int phase = 1; phase <= 3; ++phase) {
         plan.phase = phase;
-        const int rc = phase == 2  // operands and results are fp32 products inside `out`
-                           ? launch_mfma_cot<float, D, RT, CB, false, 2>(out, out, nullptr, nullptr, B, K, stream, plan)
-                           : launch_mfma_cot<Tin, D, RT, CB, false, 1>(mats, out, nullptr, nullptr, B, K, stream, plan);
+        int rc = LBI_OK;
+        if (phase != 2) {
+            rc = launch_mfma_cot<Tin, D, RT, CB, false, 1>(mats, out, nullptr, nullptr, B, K, stream, plan);
+        } else if (!log_depth) {  // operands and results are fp32 products inside `out`
+            rc = launch_mfma_cot<float, D, RT, CB, false, 2>(out, out, nullptr, nullptr, B, K, stream, plan);
+        } else {
+            plan.rd = 1;
+            for (int l = 0; l < levels && !rc; ++l) {
+                plan.off = 1 << l;
+                plan.wr = l == levels - 1 ? 0 : 3 - plan.rd;
+                rc = launch_mfma_cot<float, D, RT, CB, false, 3>(out, out, nullptr, nullptr, B, K, stream, plan);
+                plan.rd = plan.wr;
+            }
+        }
         if (rc) return rc;
     }
     if (cot) return launch_suffix_apply(out, g, cot, B, K + 1, D, stream);
@@ -823,7 +890,7 @@ template <typename Tin>
 int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, int K, int d, hipStream_t stream) {
     // Few batch elements: one chain per column block leaves most of the chip idle for K - 1 dependent steps, so
     // the chain is cut into chunks that run side by side (ScanPlan), on narrow column blocks (short steps).
-    ScanPlan plan{0, 0, 0};
+    ScanPlan plan{0, 0, 0, 0, 0, 0};
     switch (d) {
         case 256:
             if (plan_chunks(B, K, 8, &plan)) return launch_chunked<Tin, 256, 32, 32>(mats, out, g, cot, B, K, plan, stream);

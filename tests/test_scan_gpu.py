@@ -267,10 +267,13 @@ def test_k_parallel_scan_shapes(shape, dtype, device):
     assert float(torch.sqrt((((cot.cpu().double() - want) / scale) ** 2).mean())) <= 1e-5
 
 
-@pytest.mark.parametrize("chunk", [0, 2, 3, 5, 16])
-def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, device):
+@pytest.mark.parametrize("chunk,totals_chain", [(0, 0), (2, 0), (3, 0), (5, 0), (16, 0), (3, 1), (5, 1)])
+def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, totals_chain, device):
     """LBI_SCAN_CHUNK forces the chunk length (0: the plain chain): every cut of K=13 / 33 / 64, including a
-    one-matrix last chunk, meets the bar, with and without the cotangent chain."""
+    one-matrix last chunk, meets the bar, with and without the cotangent chain.  The products of the chunk totals
+    are formed in log depth where there are eight chunks or more and chunks of three matrices or more (chunk
+    lengths 3 and 5 at K = 33 / 64 here; length 3 uses the last free slot of a chunk), as one chain otherwise;
+    LBI_SCAN_TOTALS_CHAIN=1 forces the chain."""
     import os
     import subprocess
     import sys
@@ -291,7 +294,7 @@ def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, device):
         "    worst = max(worst, float(((cot.cpu().double() - c).abs() / c.abs().amax(2, keepdim=True)).max()))\n"
         "print(worst); sys.exit(0 if 0.0 < worst <= 1e-5 else 1)"
     ) % str(Path(__file__).resolve().parents[1])
-    env = dict(os.environ, LBI_SCAN_CHUNK=str(chunk))
+    env = dict(os.environ, LBI_SCAN_CHUNK=str(chunk), LBI_SCAN_TOTALS_CHAIN=str(totals_chain))
     res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert res.returncode == 0, res.stdout + res.stderr
 
