@@ -930,6 +930,12 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
                     std::getenv("LBI_SCAN_SPLIT_FP32") && std::atoi(std::getenv("LBI_SCAN_SPLIT_FP32"));
                 if (split_fp32) return scan_split::launch<Tin>(mats, out, g, cot, B, K, 3, stream);
             }
+            {
+                // Up to 32 batch elements the 64-wide blocks leave half the CUs or more without a workgroup: blocks
+                // of 32 columns (twice the workgroups, half the step time).
+                static const int narrow = std::getenv("LBI_SCAN_NARROW") ? std::atoi(std::getenv("LBI_SCAN_NARROW")) : -1;
+                if (narrow < 0 ? B <= 32 : narrow != 0) return launch_mfma<Tin, 256, 32, 32>(mats, out, g, cot, B, K, stream);
+            }
             return launch_mfma<Tin, 256, 32, 64>(mats, out, g, cot, B, K, stream);
         }
         // Column blocks of one batch element read the same matrices.  With few batch elements, narrow blocks give

@@ -22,6 +22,7 @@ SHAPES = [
     (1, 3, 300), (2, 3, 512), (1, 2, 384),  # the widest matrix-core kernel, directly and through padding
     (1, 2, 520), (2, 5, 12),  # widths the scalar kernel still runs: past the largest matrix-core width, and tiny
     (17, 2, 256), (1, 1, 256), (2, 0, 32),
+    (24, 14, 256), (33, 3, 256),  # d=256: 32-wide column blocks up to 32 batch elements, 64-wide beyond
 ]
 
 
