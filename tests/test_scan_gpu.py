@@ -268,6 +268,25 @@ def test_k_parallel_scan_shapes(shape, dtype, device):
     assert float(torch.sqrt((((cot.cpu().double() - want) / scale) ** 2).mean())) <= 1e-5
 
 
+@pytest.mark.parametrize("shape", [(1, 1000, 64), (1, 520, 256), (3, 300, 128)])
+def test_k_parallel_scan_long_chains(shape, device):
+    """Chains of hundreds of matrices (many chunks: five or six levels over the chunk totals) on the benchmark's
+    near-identity inputs: every product against the fp64 sequential product, the identity tail, reruns bit for
+    bit, and the fused cotangents against the fp64 chain."""
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks, suffix_scan_pullbacks_and_cotangents
+
+    bsz, count, rank = shape
+    mats, g = oscan.make_scan_inputs(bsz, count, rank, kind="near_identity", seed=9)
+    out, cot = suffix_scan_pullbacks_and_cotangents(mats.to(device), g.to(device))
+    truth = oscan.suffix_scan_sequential(mats, dtype=torch.float64)
+    assert torch.equal(out[:, count].cpu(), torch.eye(rank).expand(bsz, rank, rank))
+    assert _rel_err(out.cpu(), truth) <= 1e-5
+    assert torch.equal(out, suffix_scan_pullbacks(mats.to(device)))
+    want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+    scale = want.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+    assert float(((cot.cpu().double() - want).abs() / scale).max()) <= 3e-5
+
+
 @pytest.mark.parametrize("chunk,totals_chain", [(0, 0), (2, 0), (3, 0), (5, 0), (16, 0), (3, 1), (5, 1)])
 def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, totals_chain, device):
     """LBI_SCAN_CHUNK forces the chunk length (0: the plain chain): every cut of K=13 / 33 / 64, including a
