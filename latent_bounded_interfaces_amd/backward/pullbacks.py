@@ -155,14 +155,21 @@ class TorchGraphInterfacePullbackProvider:
     def __init__(self, *, basis_chunk: int = 1) -> None:
         self.basis_chunk = int(basis_chunk)
 
-    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
+    #: see ``StructuredInterfacePullbackProvider.can_skip_last_region``
+    can_skip_last_region = True
+
+    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any],
+                                     skip_last: bool = False) -> list[torch.Tensor]:
         states = cache["states"]
         if len(states) != model.num_regions + 1:
             raise ValueError("cache has invalid states length.")
         result = []
-        for s_in, s_out in zip(states[:-1], states[1:]):
+        for index, (s_in, s_out) in enumerate(zip(states[:-1], states[1:])):
             if s_in.dim() != 2 or s_out.dim() != 2:
                 raise ValueError("interface states must be [B, R].")
+            if skip_last and index == len(states) - 2:
+                result.append(None)  # never read by the scan backward step
+                break
             bsz, rank = s_out.shape
             eye = torch.eye(rank, device=s_out.device, dtype=s_out.dtype)
 
@@ -199,14 +206,21 @@ class TorchRecomputeInterfacePullbackProvider:
                                                                region_index=region_index)
         return model.interface.update(state, region_output, region_index).state
 
-    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
+    #: see ``StructuredInterfacePullbackProvider.can_skip_last_region``
+    can_skip_last_region = True
+
+    def materialize_state_jacobian_t(self, *, model: Any, cache: dict[str, Any],
+                                     skip_last: bool = False) -> list[torch.Tensor]:
         if self.basis_chunk <= 0:
             raise ValueError("basis_chunk must be > 0.")
         region_caches = cache["region_caches"]
         if len(region_caches) != model.num_regions:
             raise ValueError("cache has invalid region_caches length.")
         result = []
-        for rc in region_caches:
+        for index, rc in enumerate(region_caches):
+            if skip_last and index == len(region_caches) - 1:
+                result.append(None)  # never read by the scan backward step
+                break
             state, canvas = rc.state_in.detach(), rc.canvas_features.detach()
             if state.dim() != 2:
                 raise ValueError("interface state inputs must be [B, R].")

@@ -35,6 +35,21 @@ def test_autograd_pullback_providers_match_the_oracle_graph_provider(mode, chunk
         assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)
 
 
+@pytest.mark.parametrize("mode", ["graph", "recompute"])
+def test_autograd_pullback_providers_can_leave_out_the_last_region(mode):
+    """``skip_last=True`` (what the scan backward step of this package asks for when nothing reads the last
+    region's Jacobian): the same matrices, ``None`` in the last place."""
+    model = _model()
+    ids, _ = _batch()
+    _, cache = model.forward_with_cache(ids)
+    provider = backward.build_interface_pullback_provider(mode)
+    assert provider.can_skip_last_region
+    full = provider.materialize_state_jacobian_t(model=model, cache=cache)
+    short = provider.materialize_state_jacobian_t(model=model, cache=cache, skip_last=True)
+    assert len(short) == len(full) == 3 and short[-1] is None
+    assert all(torch.equal(a, b) for a, b in zip(short[:-1], full[:-1]))
+
+
 def test_pullback_provider_errors():
     model = _model()
     ids, _ = _batch()
