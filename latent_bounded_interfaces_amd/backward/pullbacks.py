@@ -263,3 +263,7 @@ def build_interface_pullback_provider(mode: str, *, basis_chunk: int | None = No
         return TorchRecomputeInterfacePullbackProvider(basis_chunk=basis_chunk)
     raise ValueError("interface pullback provider must be one of: graph, recompute, torch_graph, torch_recompute, "
                      "structured, hip")
+
+
+__all__ = ["StructuredInterfacePullbackProvider", "TorchGraphInterfacePullbackProvider",
+           "TorchRecomputeInterfacePullbackProvider", "build_interface_pullback_provider"]

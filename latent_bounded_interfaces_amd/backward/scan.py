@@ -170,4 +170,21 @@ class ScanADEngine:
 # The reference names the same class by its role as well (backward/scan.py:170-171).
 ReferenceScanEngine = ScanADEngine
 
-__all__ = ["LBIBackwardResult", "ReferenceScanEngine", "ScanADEngine", "lbi_scan_backward_step"]
+
+def lbi_reference_scan_backward_step(model: Any, *, ce_loss: torch.Tensor, cache: dict[str, Any],
+                                     state_jacobian_mode: str = "graph", state_jacobian_basis_chunk: int = 1,
+                                     compute_interface_jacobian_stats: bool = False,
+                                     include_interface_jacobian_suffix: bool = False) -> LBIBackwardResult:
+    """The step configured by mode name (reference backward/reference_scan.py:12-34: same keywords and defaults):
+    the provider comes from ``build_interface_pullback_provider``, the local VJPs from the default autograd
+    provider.  Besides the reference's ``graph`` / ``recompute``, ``structured`` selects the provider whose region
+    pullback runs on the HIP kernels (``state_jacobian_basis_chunk`` then counts directions per call, 0 = all)."""
+    return lbi_scan_backward_step(
+        model, ce_loss=ce_loss, cache=cache,
+        pullback_provider=build_interface_pullback_provider(state_jacobian_mode, basis_chunk=state_jacobian_basis_chunk),
+        compute_interface_jacobian_stats=compute_interface_jacobian_stats,
+        include_interface_jacobian_suffix=include_interface_jacobian_suffix)
+
+
+__all__ = ["LBIBackwardResult", "ReferenceScanEngine", "ScanADEngine", "lbi_reference_scan_backward_step",
+           "lbi_scan_backward_step"]

@@ -185,3 +185,8 @@ def interface_state_jacobian_t_stats(
             keys += ["jac_suffix_spec_mean", "jac_suffix_spec_max"]
         host = torch.stack(values).cpu().tolist()
         return dict(zip(keys, (float(v) for v in host)))
+
+
+__all__ = ["apply_jacobian_t", "compose_suffix_jacobian_t", "interface_state_jacobian_t_stats",
+           "propagate_state_adjoint_by_autograd_chain", "propagate_state_adjoint_from_last_region_input",
+           "propagate_state_adjoint_with_jacobian_scan"]
