@@ -11,7 +11,8 @@ from typing import Any
 import torch
 
 from ..hip.transformer import attention_input_pullback_basis as hip_attention_input_pullback_basis
-from ..hip.transformer.region import region_input_pullback_basis, region_parameter_vjp
+from ..hip.transformer.region import (region_input_pullback_basis, region_parameter_vjp,
+                                      region_parameter_vjp_with_input_cotangent)
 
 
 class HipTransformerLowering:
@@ -35,9 +36,11 @@ class HipTransformerLowering:
         output_cotangent_basis: torch.Tensor,
         softmax_scale: float,
         causal: bool = True,
-        kernel_mode: str = "hip",
+        kernel_mode: str = "fa2_mma_pblock4",
     ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-        """Same keyword-only contract as reference backends/transformer_cuda.py:23-43."""
+        """Same keyword-only contract and default mode as reference backends/transformer_cuda.py:23-43 (the
+        default therefore keeps that mode's limit of four directions per call, a ``ValueError`` beyond it);
+        ``kernel_mode="hip"`` is the mode without a limit.  Every mode runs the same HIP kernels."""
         return hip_attention_input_pullback_basis(
             q,
             k,
@@ -69,3 +72,13 @@ class HipTransformerLowering:
         if self.reference_lowering is not None:
             return self.reference_lowering.parameter_vjp(backend=backend, cache=cache, output_cotangent=output_cotangent)
         return region_parameter_vjp(backend, cache, output_cotangent, kernel_mode="hip")
+
+    def parameter_vjp_with_input_cotangent(self, *, backend: Any, cache: Any, output_cotangent: torch.Tensor
+                                           ) -> tuple[dict[str, torch.Tensor], torch.Tensor]:
+        """``parameter_vjp`` plus the cotangent of the region input ``[B, T, D]`` (fp32) from the same sweep; not
+        part of the reference's lowering protocol, used by ``StructuredLocalVJPProvider`` when present."""
+        if self.reference_lowering is not None:
+            grads = self.reference_lowering.parameter_vjp(backend=backend, cache=cache, output_cotangent=output_cotangent)
+            g_in = region_input_pullback_basis(backend, cache, output_cotangent.unsqueeze(1), kernel_mode="hip")[:, 0]
+            return grads, g_in
+        return region_parameter_vjp_with_input_cotangent(backend, cache, output_cotangent, kernel_mode="hip")

@@ -27,6 +27,8 @@ from typing import Any
 
 import torch
 
+from ..contracts import InterfacePullbackProvider
+
 
 class StructuredInterfacePullbackProvider:
     """Builds ``Jt`` per region from the interface's and the backend's structured pullbacks."""
@@ -244,6 +246,22 @@ class TorchRecomputeInterfacePullbackProvider:
         return result
 
 
+def materialize_interface_state_jacobian_t_graph(*, model: Any, cache: dict[str, Any]) -> list[torch.Tensor]:
+    """Function form of the graph provider (reference backward/pullbacks.py:37-81)."""
+    return TorchGraphInterfacePullbackProvider().materialize_state_jacobian_t(model=model, cache=cache)
+
+
+def materialize_interface_state_jacobian_t_recompute(*, model: Any, cache: dict[str, Any],
+                                                     basis_chunk: int = 1) -> list[torch.Tensor]:
+    """Function form of the recompute provider (reference backward/pullbacks.py:84-149)."""
+    return TorchRecomputeInterfacePullbackProvider(basis_chunk=basis_chunk).materialize_state_jacobian_t(
+        model=model, cache=cache)
+
+
+#: normalised mode names that select the structured provider
+STRUCTURED_MODE_NAMES = frozenset({"structured", "hip", "structured_hip"})
+
+
 def build_interface_pullback_provider(mode: str, *, basis_chunk: int | None = None,
                                       position_constant_update: str = "verify_once"):
     """Provider by name.  ``graph`` / ``recompute`` and their aliases are the reference's modes
@@ -253,7 +271,7 @@ def build_interface_pullback_provider(mode: str, *, basis_chunk: int | None = No
     ``basis_chunk=None`` means the reference's default of 1 for the autograd providers and 0 (all ``d``
     directions in one call) for the structured one."""
     normalized = str(mode).strip().lower().replace("-", "_")
-    if normalized in {"structured", "hip", "structured_hip"}:
+    if normalized in STRUCTURED_MODE_NAMES:
         return StructuredInterfacePullbackProvider(basis_chunk=0 if basis_chunk is None else basis_chunk,
                                                    position_constant_update=position_constant_update)
     basis_chunk = 1 if basis_chunk is None else basis_chunk
@@ -265,5 +283,7 @@ def build_interface_pullback_provider(mode: str, *, basis_chunk: int | None = No
                      "structured, hip")
 
 
-__all__ = ["StructuredInterfacePullbackProvider", "TorchGraphInterfacePullbackProvider",
-           "TorchRecomputeInterfacePullbackProvider", "build_interface_pullback_provider"]
+__all__ = ["InterfacePullbackProvider", "STRUCTURED_MODE_NAMES", "StructuredInterfacePullbackProvider",
+           "TorchGraphInterfacePullbackProvider", "TorchRecomputeInterfacePullbackProvider",
+           "build_interface_pullback_provider", "materialize_interface_state_jacobian_t_graph",
+           "materialize_interface_state_jacobian_t_recompute"]

@@ -5,18 +5,18 @@ Counterparts of ``lbi_scan_backward_step`` and ``ScanADEngine`` / ``ReferenceSca
 keys, same order of calls into the local-VJP provider, same edge cases (no region:
 ``RuntimeError``; one region: no Jacobian is built).  What differs is the middle:
 
-* the state adjoints and the suffix matrices come from ONE launch
-  (``lbi_suffix_scan_with_cotangents``): the adjoints are the chain ``g_r = Jt_r g_{r+1}`` carried
-  beside the matrix products;
+* the state adjoints are every suffix matrix applied to the last cotangent in ONE launch
+  (``lbi_suffix_apply``; the reference spends K mat-vec launches, backward/suffix_scan.py:49-53);
 * the last region's state Jacobian, which the reference builds and then drops (its output state never reaches the
   loss), is not built when the provider can leave it out and the Jacobian statistics are off: one region pullback
   less per step;
 * ``interface_scan_rms`` (logged by the reference's training loop as ``scan_align``) is reported
-  on every step as the reference does (:63-72), from the two independent results that launch
-  yields: the chain, and the suffix matrices applied to the last cotangent (one more launch
-  for all regions together, one reduction, one scalar read - where the reference spends K
-  mat-vec launches and the same read).  ``check_scan=False`` skips it (no suffix matrix is formed,
-  no host synchronisation, 0.0 reported) for callers that do not log it.
+  on every step as the reference does (:63-72): the RMS difference between those adjoints and the
+  sequential chain ``g_r = Jt_r g_{r+1}`` (the reference's ``g_manual``), which comes from a kernel of its
+  own (``lbi_suffix_cotangents``: one pass over the matrices, no matrix product).  The two sides share no
+  intermediate result whatever form the scan takes (one chain per column block, or chunks side by side),
+  so the figure checks the scan and is tiny but not zero.  ``check_scan=False`` skips it (no suffix
+  matrix is formed, no host synchronisation, 0.0 reported) for callers that do not log it.
 """
 from __future__ import annotations
 
@@ -25,10 +25,10 @@ from typing import Any
 import torch
 from torch import nn
 
-from ..hip.interface import suffix_apply, suffix_scan_pullbacks_and_cotangents
+from ..hip.interface import suffix_apply, suffix_scan_cotangents, suffix_scan_pullbacks
 from .base import ADResult, LBIBackwardResult, ScanBackpropModel, assign_grad_map
-from .local_vjp import TorchAutogradLocalVJPProvider
-from .pullbacks import build_interface_pullback_provider
+from .local_vjp import TorchAutogradLocalVJPProvider, build_local_vjp_provider
+from .pullbacks import STRUCTURED_MODE_NAMES, build_interface_pullback_provider
 from .suffix_scan import (
     _stack_for_chain,
     interface_state_jacobian_t_stats,
@@ -40,12 +40,14 @@ def _adjoints_and_scan_rms(state_jacobians_t, g_last_input: torch.Tensor) -> tup
     """State adjoints of every region input plus the RMS difference between the two ways of getting them."""
     stacked = _stack_for_chain(state_jacobians_t[:-1])            # the last region's output state is unused
     count = stacked.shape[1]
-    suffix, chain = suffix_scan_pullbacks_and_cotangents(stacked, g_last_input)
-    # suffix[b, r] @ g[b] for all (b, r) at once (the identity tail returns g, as the chain does)
-    applied = suffix_apply(suffix, g_last_input)
+    # suffix[b, r] @ g[b] for all (b, r) at once (the identity tail returns g): the adjoints the step uses,
+    # formed the way the reference forms them (backward/suffix_scan.py:49-53)
+    applied = suffix_apply(suffix_scan_pullbacks(stacked), g_last_input)
+    # the sequential chain from a kernel that shares nothing with the scan (the reference's g_manual, :63-69)
+    chain = suffix_scan_cotangents(stacked, g_last_input)
     # mean over the count + 1 regions of the per-region mean square
     rms = torch.sqrt(((applied - chain) ** 2).mean())
-    adjoints = [chain[:, r].to(g_last_input.dtype) for r in range(count + 1)]
+    adjoints = [applied[:, r].to(g_last_input.dtype) for r in range(count + 1)]
     return adjoints, float(rms.item())
 
 
@@ -62,6 +64,9 @@ def lbi_scan_backward_step(
 ) -> LBIBackwardResult:
     """Exact scan backward for an LBI model using a supplied interface-pullback provider."""
     local_vjp_provider = local_vjp_provider or TorchAutogradLocalVJPProvider()
+    bind_cache = getattr(local_vjp_provider, "bind_cache", None)
+    if bind_cache is not None:
+        bind_cache(cache)                # a provider that works from the cache (the protocol's calls do not pass it)
     grad_map = local_vjp_provider.new_grad_map(model)
     states = list(cache["states"])
     num_regions = len(list(cache["region_ranges"]))
@@ -119,24 +124,40 @@ class ScanADEngine:
         pullback_provider: Any | None = None,
         local_vjp_provider: Any | None = None,
         state_jacobian_mode: str = "graph",
-        state_jacobian_basis_chunk: int = 1,
+        state_jacobian_basis_chunk: int | None = None,
         compute_interface_jacobian_stats: bool = False,
         include_interface_jacobian_suffix: bool = False,
+        local_vjp_mode: str = "autograd",
     ) -> None:
+        # ``state_jacobian_basis_chunk=None``: the provider's own default, which is the reference's 1 for its
+        # autograd modes and "all d directions in one call" for the structured provider
+
         self.pullback_provider = pullback_provider or build_interface_pullback_provider(
             state_jacobian_mode, basis_chunk=state_jacobian_basis_chunk)
-        self.local_vjp_provider = local_vjp_provider or TorchAutogradLocalVJPProvider()
+        # ``local_vjp_mode="structured"``: region parameter VJPs on the HIP kernels instead of the forward graph
+        self.local_vjp_provider = local_vjp_provider or build_local_vjp_provider(local_vjp_mode)
         self.compute_interface_jacobian_stats = bool(compute_interface_jacobian_stats)
         self.include_interface_jacobian_suffix = bool(include_interface_jacobian_suffix)
 
     @classmethod
     def from_config(cls, cfg: Any, *, compute_interface_jacobian_stats: bool = False) -> "ScanADEngine":
         """Reads ``interface_jacobian_mode``, ``jacobian_basis_chunk`` and ``log_interface_jacobian_suffix``
-        of the reference's training configuration (train/config.py:164-171)."""
+        of the reference's training configuration (train/config.py:164-171).
+
+        ``jacobian_basis_chunk`` is the reference's memory knob for its autograd providers (copies of the batch
+        per recompute pass; default 1, values <= 0 rejected by its validator, train/config.py:169, :330) and is
+        passed to those only.  The structured provider has no replicated batch: it pulls all ``d`` directions
+        back in one call per region unless the configuration carries ``structured_basis_chunk`` (directions per
+        call; absent or 0 = all), so a reference configuration object with its defaults gets the fast form.
+        ``local_vjp_mode`` (absent = ``autograd``, the reference's provider) selects the local-VJP provider."""
+        mode = str(cfg.interface_jacobian_mode)
+        if mode.strip().lower().replace("-", "_") in STRUCTURED_MODE_NAMES:
+            chunk = int(getattr(cfg, "structured_basis_chunk", 0) or 0)
+        else:
+            chunk = int(cfg.jacobian_basis_chunk)
         return cls(
-            pullback_provider=build_interface_pullback_provider(
-                str(cfg.interface_jacobian_mode), basis_chunk=int(cfg.jacobian_basis_chunk)),
-            local_vjp_provider=TorchAutogradLocalVJPProvider(),
+            pullback_provider=build_interface_pullback_provider(mode, basis_chunk=chunk),
+            local_vjp_provider=build_local_vjp_provider(str(getattr(cfg, "local_vjp_mode", "autograd"))),
             compute_interface_jacobian_stats=compute_interface_jacobian_stats,
             include_interface_jacobian_suffix=bool(cfg.log_interface_jacobian_suffix),
         )
@@ -172,13 +193,16 @@ ReferenceScanEngine = ScanADEngine
 
 
 def lbi_reference_scan_backward_step(model: Any, *, ce_loss: torch.Tensor, cache: dict[str, Any],
-                                     state_jacobian_mode: str = "graph", state_jacobian_basis_chunk: int = 1,
+                                     state_jacobian_mode: str = "graph",
+                                     state_jacobian_basis_chunk: int | None = None,
                                      compute_interface_jacobian_stats: bool = False,
                                      include_interface_jacobian_suffix: bool = False) -> LBIBackwardResult:
-    """The step configured by mode name (reference backward/reference_scan.py:12-34: same keywords and defaults):
+    """The step configured by mode name (reference backward/reference_scan.py:12-34: same keywords):
     the provider comes from ``build_interface_pullback_provider``, the local VJPs from the default autograd
     provider.  Besides the reference's ``graph`` / ``recompute``, ``structured`` selects the provider whose region
-    pullback runs on the HIP kernels (``state_jacobian_basis_chunk`` then counts directions per call, 0 = all)."""
+    pullback runs on the HIP kernels (``state_jacobian_basis_chunk`` then counts directions per call, 0 = all).
+    ``state_jacobian_basis_chunk=None`` is the reference's default of 1 for its own modes and all directions in
+    one call for ``structured``."""
     return lbi_scan_backward_step(
         model, ce_loss=ce_loss, cache=cache,
         pullback_provider=build_interface_pullback_provider(state_jacobian_mode, basis_chunk=state_jacobian_basis_chunk),

@@ -39,7 +39,7 @@ class TransformerLowering(Protocol):
 
     def attention_input_pullback_basis(self, *, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                                        output_cotangent_basis: torch.Tensor, softmax_scale: float,
-                                       causal: bool = True, kernel_mode: str = "hip"
+                                       causal: bool = True, kernel_mode: str = "fa2_mma_pblock4"
                                        ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]: ...
 
     def input_pullback_basis(self, *, backend: Any, cache: Any, output_cotangent_basis: torch.Tensor

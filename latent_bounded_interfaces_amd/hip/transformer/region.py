@@ -449,16 +449,11 @@ def region_input_pullback_basis(backend: Any, cache: Any, output_cotangent_basis
         return g.to(device=output_cotangent_basis.device, dtype=output_cotangent_basis.dtype)
 
 
-def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tensor, *,
-                         kernel_mode: str = "hip") -> dict[str, torch.Tensor]:
-    """Parameter gradients of one region for ``output_cotangent [B, T, D]``, keyed by the
-    parameter names of ``backend.named_parameters()``.
-
-    ``TransformerLowering.parameter_vjp`` of the reference (backends/transformer.py:76-85;
-    autograd version :332-355).  One backward sweep over the cached activations with a single
-    direction; every weight gradient is a plain GEMM of the cotangent at a module's output
-    with the module's cached input.
-    """
+def region_parameter_vjp_with_input_cotangent(backend: Any, cache: Any, output_cotangent: torch.Tensor, *,
+                                              kernel_mode: str = "hip") -> tuple[dict[str, torch.Tensor], torch.Tensor]:
+    """:func:`region_parameter_vjp` together with the cotangent of the region input ``[B, T, D]`` (fp32) that the
+    same backward sweep ends with: what a local-VJP provider needs to carry a region's seed on to the decoder of
+    the interface and to the canvas, at no extra cost."""
     if output_cotangent.dim() != 3:
         raise ValueError("output_cotangent must have shape [B, T, D]")
     if not output_cotangent.is_cuda:
@@ -469,17 +464,32 @@ def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tenso
     by_id: dict[int, torch.Tensor] = {}
     if end > start:
         with torch.no_grad():
-            _pull_back_region(backend, cache, output_cotangent.unsqueeze(1), kernel_mode, by_id)
+            g_input = _pull_back_region(backend, cache, output_cotangent.unsqueeze(1), kernel_mode, by_id)[:, 0]
+    else:
+        g_input = output_cotangent.detach().float()
     wanted = {id(p) for layer_cache in cache.layer_caches
               for p in backend.backbone.blocks[layer_cache.layer_index].parameters() if p.requires_grad}
     out: dict[str, torch.Tensor] = {}
     for name, param in backend.named_parameters():
         if id(param) in wanted and id(param) in by_id:
             out[name] = by_id[id(param)].detach()
-    return out
+    return out, g_input
+
+
+def region_parameter_vjp(backend: Any, cache: Any, output_cotangent: torch.Tensor, *,
+                         kernel_mode: str = "hip") -> dict[str, torch.Tensor]:
+    """Parameter gradients of one region for ``output_cotangent [B, T, D]``, keyed by the
+    parameter names of ``backend.named_parameters()``.
+
+    ``TransformerLowering.parameter_vjp`` of the reference (backends/transformer.py:76-85;
+    autograd version :332-355).  One backward sweep over the cached activations with a single
+    direction; every weight gradient is a plain GEMM of the cotangent at a module's output
+    with the module's cached input.
+    """
+    return region_parameter_vjp_with_input_cotangent(backend, cache, output_cotangent, kernel_mode=kernel_mode)[0]
 
 
 __all__ = [
     "attn_heads_split", "attn_qkv_conv_pullback", "attn_qkv_pullback", "causal_conv1d_pullback",
-    "causal_conv1d_weight_grad", "gated_mlp_pullback", "rmsnorm_pullback", "rmsnorm_weight_grad", "region_input_pullback_basis", "region_parameter_vjp", "rope_tables",
+    "causal_conv1d_weight_grad", "gated_mlp_pullback", "rmsnorm_pullback", "rmsnorm_weight_grad", "region_input_pullback_basis", "region_parameter_vjp", "region_parameter_vjp_with_input_cotangent", "rope_tables",
 ]

@@ -128,6 +128,11 @@ class _BackendWithLowering(oreg.OracleRegionBackend):
             return oreg.input_pullback_basis_autograd(self, cache, output_cotangent_basis)
         return self.lowering.input_pullback_basis(backend=self, cache=cache, output_cotangent_basis=output_cotangent_basis)
 
+    def parameter_vjp(self, *, cache, output_cotangent):
+        if self.lowering is None:
+            return oreg.parameter_vjp_autograd(self, cache, output_cotangent)
+        return self.lowering.parameter_vjp(backend=self, cache=cache, output_cotangent=output_cotangent)
+
 
 class OracleLBIModel(nn.Module):
     def __init__(self, *, vocab_size, dim, n_heads, layers, layers_per_region, interface_width, n_kv_heads=None,
@@ -186,6 +191,25 @@ class OracleLBIModel(nn.Module):
                         "region_inputs": [rc.region_input for rc in region_caches],
                         "region_outputs": [rc.region_output for rc in region_caches],
                         "region_ranges": self.region_ranges, "region_caches": region_caches}
+
+
+#: the end-to-end benchmark configuration: 12 layers, d_model 768, 12 heads of 64, vocabulary 50257, 6 regions of
+#: 2 layers, vector-MLP interface of width 64 (16-bit weights and activations, fp32 interface), batch 8, T 1024
+END_TO_END = dict(vocab_size=50257, dim=768, n_heads=12, n_kv_heads=12, layers=12, layers_per_region=2,
+                  interface_width=64, hidden=3072, d_conv=4, interface_hidden=0)
+END_TO_END_BATCH, END_TO_END_SEQ = 8, 1024
+
+
+def end_to_end_model(*, dtype=torch.bfloat16, lowering=None, seed=0, **overrides) -> "OracleLBIModel":
+    """The stand-in model at the end-to-end configuration (random init from a fixed seed)."""
+    return OracleLBIModel(**{**END_TO_END, **overrides}, lowering=lowering, dtype=dtype, seed=seed)
+
+
+def end_to_end_batch(*, batch=END_TO_END_BATCH, seq_len=END_TO_END_SEQ, vocab_size=END_TO_END["vocab_size"], seed=0):
+    """Token ids and targets, uniform over the vocabulary, from a CPU generator."""
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randint(0, vocab_size, (batch, seq_len), generator=gen),
+            torch.randint(0, vocab_size, (batch, seq_len), generator=gen))
 
 
 def token_loss(logits: torch.Tensor, targets: torch.Tensor) -> torch.Tensor:

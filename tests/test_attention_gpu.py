@@ -163,7 +163,14 @@ def test_modes_and_contract(device):
     # lowering wrapper (reference tests/test_cuda_attention_pullback.py:294-315)
     low = HipTransformerLowering()
     assert low.name == "hip"
-    out = low.attention_input_pullback_basis(q=q, k=k, v=v, output_cotangent_basis=g5, softmax_scale=scale)
+    out = low.attention_input_pullback_basis(q=q, k=k, v=v, output_cotangent_basis=g, softmax_scale=scale)
+    assert all(torch.equal(a, b) for a, b in zip(out, base))
+    # the default mode is the reference's (backends/transformer_cuda.py:31) with its limit of four directions;
+    # "hip" is the mode without one
+    with pytest.raises(ValueError, match="<= 4"):
+        low.attention_input_pullback_basis(q=q, k=k, v=v, output_cotangent_basis=g5, softmax_scale=scale)
+    out = low.attention_input_pullback_basis(q=q, k=k, v=v, output_cotangent_basis=g5, softmax_scale=scale,
+                                             kernel_mode="hip")
     assert all(torch.equal(a[:, :4], b) for a, b in zip(out, base))
     with pytest.raises(RuntimeError, match="no CPU execution path"):
         low.input_pullback_basis(backend=None, cache=None, output_cotangent_basis=torch.zeros(1, 1, 2, 3))

@@ -83,6 +83,79 @@ def test_default_local_vjp_provider_reproduces_dense_gradients(layers, per_regio
             assert torch.allclose(grads[name], want.to(grads[name].dtype), atol=1e-6, rtol=1e-4), (name, float((grads[name] - want).abs().max()))
 
 
+@pytest.mark.parametrize("layers,per_region", [(3, 1), (4, 2), (2, 2)])
+def test_structured_local_vjp_provider_reproduces_dense_gradients(layers, per_region):
+    """The cache-based local-VJP provider, with the region sweeps answered by autograd of the oracle region (the
+    two-call form of the lowering protocol) so that it runs without a GPU: the gradient map of the scan step equals
+    ``loss.backward()`` of the same graph (fp64 apart from the norm, which the oracle block runs in fp32), name by name, ``None`` where the dense path leaves ``None``."""
+    model = _model(layers=layers, layers_per_region=per_region)
+    ids, targets = _batch()
+    _, dense = olbi.dense_gradients(model, ids, targets)
+    logits, cache = model.forward_with_cache(ids)
+    provider = backward.StructuredLocalVJPProvider(cache=cache)
+    assert isinstance(provider, backward.LocalVJPProvider) and provider.name == "structured"
+    grads = olbi.scan_backward_step_sequential(
+        model, loss=olbi.token_loss(logits, targets), cache=cache,
+        pullback_provider=backward.TorchGraphInterfacePullbackProvider(), local_vjp_provider=provider)
+    assert set(grads) == set(dense)
+    for name, want in dense.items():
+        if want is None:
+            assert grads[name] is None, name
+        else:
+            assert grads[name] is not None, name
+            assert torch.allclose(grads[name], want, atol=1e-7, rtol=1e-5), (name, float((grads[name] - want).abs().max()))
+
+
+def test_structured_local_vjp_provider_contract():
+    model = _model()
+    ids, targets = _batch()
+    logits, cache = model.forward_with_cache(ids)
+    loss = olbi.token_loss(logits, targets)
+    unbound = backward.StructuredLocalVJPProvider()
+    with pytest.raises(RuntimeError, match="forward cache"):
+        unbound.store_output_head_grads(model=model, loss=loss, grad_map={})
+    unbound.bind_cache(cache)
+    # a state other than the one the last region read is answered by the graph
+    unbound.store_output_head_grads(model=model, loss=loss, grad_map=unbound.new_grad_map(model))
+    want = torch.autograd.grad(loss, cache["states"][0], retain_graph=True)[0]
+    assert torch.equal(unbound.state_adjoint_from_loss(loss=loss, state=cache["states"][0]), want)
+    want = torch.autograd.grad(loss, cache["states"][-2], retain_graph=True)[0]
+    got = unbound.state_adjoint_from_loss(loss=loss, state=cache["states"][-2])
+    assert torch.allclose(got, want, atol=1e-12, rtol=1e-9)
+    assert backward.build_local_vjp_provider("structured").name == "structured"
+    assert backward.build_local_vjp_provider("torch-autograd").name == "torch_autograd"
+    with pytest.raises(ValueError, match="must be one of"):
+        backward.build_local_vjp_provider("dense")
+
+
+def test_package_exports_every_name_of_the_reference_package():
+    """reference backward/__init__.py:22-50."""
+    reference_names = [
+        "ADEngine", "ADResult", "AutogradEngine", "GradMap", "InterfacePullbackProvider", "LBIBackwardResult",
+        "LocalVJPProvider", "ReferenceScanEngine", "ScanADEngine", "ScanBackpropModel", "TorchAutogradLocalVJPProvider",
+        "TorchGraphInterfacePullbackProvider", "TorchRecomputeInterfacePullbackProvider", "assign_grad_map",
+        "autograd_backward_step", "apply_jacobian_t", "build_interface_pullback_provider", "collect_named_grads",
+        "compose_suffix_jacobian_t", "lbi_reference_scan_backward_step", "lbi_scan_backward_step",
+        "materialize_interface_state_jacobian_t_graph", "materialize_interface_state_jacobian_t_recompute",
+        "propagate_state_adjoint_by_autograd_chain", "propagate_state_adjoint_from_last_region_input",
+        "propagate_state_adjoint_with_jacobian_scan", "store_named_grads"]
+    assert [n for n in reference_names if n not in backward.__all__ or not hasattr(backward, n)] == []
+    model = _model()
+    ids, targets = _batch()
+    _, dense = olbi.dense_gradients(model, ids, targets)
+    logits, cache = model.forward_with_cache(ids)
+    grads = backward.autograd_backward_step(model, ce_loss=olbi.token_loss(logits, targets))
+    assert all((grads[n] is None) == (dense[n] is None) and (dense[n] is None or torch.equal(grads[n], dense[n]))
+               for n in dense)
+    assert backward.AutogradEngine.name == "autograd"
+    _, cache = model.forward_with_cache(ids)          # the dense step released the graph of the first forward
+    want = backward.TorchGraphInterfacePullbackProvider().materialize_state_jacobian_t(model=model, cache=cache)
+    got = backward.materialize_interface_state_jacobian_t_graph(model=model, cache=cache)
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
+    got = backward.materialize_interface_state_jacobian_t_recompute(model=model, cache=cache, basis_chunk=2)
+    assert all(torch.allclose(a, b, atol=1e-12) for a, b in zip(got, want))
+
+
 def test_autograd_chain_diagnostic_matches_the_jacobian_chain():
     model = _model()
     ids, targets = _batch()

@@ -399,3 +399,124 @@ def test_step_leaves_out_the_last_regions_jacobian_unless_statistics_read_it(dev
     short = provider.materialize_state_jacobian_t(model=model, cache=cache, skip_last=True)
     assert len(short) == len(full) == 3 and short[-1] is None
     assert all(torch.equal(a, b) for a, b in zip(short[:-1], full[:-1]))
+
+
+def test_scan_cross_check_compares_two_independent_results_in_the_k_parallel_form(device):
+    """With few batch elements and a long chain the scan runs its chunks side by side and forms the cotangents by
+    applying the finished products to g.  ``interface_scan_rms`` must still compare two results that share nothing:
+    the applied suffix matrices against the sequential chain of a kernel of its own, so it is tiny but not zero."""
+    from latent_bounded_interfaces_amd.backward.scan import _adjoints_and_scan_rms
+    from oracle import scan as oscan
+
+    for bsz, count, rank in ((1, 16, 64), (2, 24, 256), (4, 5, 64)):
+        mats, g = oscan.make_scan_inputs(bsz, count, rank, kind="near_identity", seed=5)
+        jts = [mats[:, r].to(device) for r in range(count)] + [torch.zeros(bsz, rank, rank, device=device)]
+        adjoints, rms = _adjoints_and_scan_rms(jts, g.to(device))
+        assert 0.0 < rms < 1e-5, (bsz, count, rank, rms)
+        want = oscan.suffix_cotangents_sequential(mats.double(), g.double())
+        assert len(adjoints) == count + 1
+        for r, a in enumerate(adjoints):
+            assert torch.allclose(a.cpu().double(), want[:, r], atol=1e-5, rtol=1e-5), (bsz, count, rank, r)
+
+
+def test_engine_from_a_reference_configuration_pulls_all_directions_back_in_one_call(device):
+    """The reference's configuration defaults ``jacobian_basis_chunk`` to 1 and rejects values <= 0
+    (train/config.py:169, :330): that knob is for its autograd providers.  ``from_config`` with
+    ``interface_jacobian_mode="structured"`` must not turn it into one region pullback per direction."""
+    from types import SimpleNamespace
+
+    from latent_bounded_interfaces_amd.backward import ScanADEngine, lbi_reference_scan_backward_step
+
+    model = _model(device)
+    cfg = SimpleNamespace(interface_jacobian_mode="structured", jacobian_basis_chunk=1,
+                          log_interface_jacobian_suffix=False)
+    engine = ScanADEngine.from_config(cfg)
+    assert engine.pullback_provider.name == "structured" and engine.pullback_provider.basis_chunk == 0
+    assert ScanADEngine(state_jacobian_mode="structured").pullback_provider.basis_chunk == 0
+    assert ScanADEngine(state_jacobian_mode="recompute").pullback_provider.basis_chunk == 1
+    assert ScanADEngine.from_config(SimpleNamespace(interface_jacobian_mode="recompute", jacobian_basis_chunk=3,
+                                                    log_interface_jacobian_suffix=False)
+                                    ).pullback_provider.basis_chunk == 3
+    cfg.structured_basis_chunk = 4
+    assert ScanADEngine.from_config(cfg).pullback_provider.basis_chunk == 4
+    calls = []
+    inner = model.region_backend.input_pullback_basis
+
+    def spy(*, cache, output_cotangent_basis):
+        calls.append((cache.region_index, int(output_cotangent_basis.shape[1])))
+        return inner(cache=cache, output_cotangent_basis=output_cotangent_basis)
+
+    model.region_backend.input_pullback_basis = spy
+    try:
+        loss, cache, dense = _step_inputs(model, device)
+        result = engine.backward(model=model, loss=loss, cache=cache)
+        assert calls == [(0, 8), (1, 8)]           # one call per region that the scan reads, all 8 directions
+        _check_grads(result.grad_map, dense)
+        calls.clear()
+        loss, cache, dense = _step_inputs(model, device)
+        lbi_reference_scan_backward_step(model, ce_loss=loss, cache=cache, state_jacobian_mode="structured")
+        assert calls == [(0, 8), (1, 8)]
+    finally:
+        del model.region_backend.input_pullback_basis
+
+
+@pytest.mark.parametrize("layers,per_region", [(6, 2), (3, 1), (2, 2)])
+def test_structured_local_vjp_provider_matches_the_autograd_provider_and_dense_gradients(layers, per_region, device):
+    """Region parameter VJPs from the forward cache on the HIP kernels (``StructuredLocalVJPProvider``) against the
+    reference's provider (autograd on the forward graph) and against ``loss.backward()``, fp32 bar of the reference
+    (tests/test_lbi_gradient_parity.py:40-41); same ``None`` pattern (parameters the loss does not reach)."""
+    from latent_bounded_interfaces_amd.backward import (ScanADEngine, StructuredInterfacePullbackProvider,
+                                                        StructuredLocalVJPProvider, lbi_scan_backward_step)
+
+    model = _model(device, layers=layers, layers_per_region=per_region)
+    loss, cache, dense = _step_inputs(model, device)
+    want = lbi_scan_backward_step(model, ce_loss=loss, cache=cache,
+                                  pullback_provider=StructuredInterfacePullbackProvider())
+    loss, cache, _ = _step_inputs(model, device)
+    got = lbi_scan_backward_step(model, ce_loss=loss, cache=cache,
+                                 pullback_provider=StructuredInterfacePullbackProvider(),
+                                 local_vjp_provider=StructuredLocalVJPProvider())
+    assert got.interface_scan_rms < 1e-5
+    _check_grads(got.grad_map, dense)
+    _check_grads(got.grad_map, want.grad_map)
+    # through the engine, by mode name, and from a configuration object
+    from types import SimpleNamespace
+
+    loss, cache, _ = _step_inputs(model, device)
+    engine = ScanADEngine(state_jacobian_mode="structured", local_vjp_mode="structured")
+    result = engine.backward(model=model, loss=loss, cache=cache)
+    assert result.diagnostics["local_vjp_provider"] == "structured"
+    _check_grads(result.grad_map, dense)
+    cfg = SimpleNamespace(interface_jacobian_mode="structured", jacobian_basis_chunk=1,
+                          log_interface_jacobian_suffix=False, local_vjp_mode="structured")
+    assert ScanADEngine.from_config(cfg).local_vjp_provider.name == "structured"
+
+
+def test_structured_local_vjp_provider_on_16bit_weights(device):
+    """bf16 weights and activations, fp32 interface, heads of 64 and T = 320 (the matrix-core attention kernels run
+    in the sweeps): against fp32 dense gradients on the same rounded weights at the reference's 16-bit bar."""
+    import copy
+
+    from latent_bounded_interfaces_amd.backward import ScanADEngine
+
+    model = _model(device, dtype=torch.bfloat16, dim=128, n_heads=2, n_kv_heads=2, hidden=256, layers=4,
+                   layers_per_region=2, interface_width=64, interface_hidden=96, seed=37)
+    dense_model = copy.deepcopy(model).float()
+    dense_model.region_backend.lowering = None
+    gen = torch.Generator().manual_seed(9)
+    ids = torch.randint(0, 61, (2, 320), generator=gen).to(device)
+    targets = torch.randint(0, 61, (2, 320), generator=gen).to(device)
+    _, dense = olbi.dense_gradients(dense_model, ids, targets)
+    logits, cache = model.forward_with_cache(ids)
+    engine = ScanADEngine(state_jacobian_mode="structured", local_vjp_mode="structured")
+    result = engine.backward(model=model, loss=olbi.token_loss(logits, targets), cache=cache)
+    params = dict(model.named_parameters())
+    for name, want in dense.items():
+        got = result.grad_map[name]
+        assert (got is None) == (want is None), name
+        if want is None:
+            continue
+        assert got.dtype == params[name].dtype and got.shape == want.shape, name
+        assert torch.allclose(got.float(), want, atol=5e-2, rtol=5e-2), (name, float((got.float() - want).abs().max()))
+        rel = float((got.float() - want).norm() / want.norm().clamp_min(1e-12))
+        assert rel <= 5e-2, (name, rel)
