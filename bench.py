@@ -14,10 +14,11 @@ Prints ONE JSON line.  Besides the contract keys it carries
 * ``cpu_baseline``  - the reference's CPU algorithm (log-depth torch scan) timed on the
                       host cores of the same box on a bounded batch slice;
 * ``extra``         - the other measured variants (bf16 storage, cotangent-only chain,
-                      attention input-pullback, region-level input pullback) with their own
-                      roofline figures; the two attention entries carry a ``cpu_baseline`` of
-                      their own (the reference's per-direction SDPA + autograd loop, fp32, on a
-                      bounded sample).
+                      attention input-pullback, region-level input pullback, the end-to-end LBI
+                      backward step on a real forward cache) with their own roofline figures; the
+                      attention and end-to-end entries carry a ``cpu_baseline`` of their own (the
+                      reference's per-direction SDPA + autograd loop, resp. dense fp32
+                      ``loss.backward()``, on a bounded sample).
 """
 from __future__ import annotations
 
@@ -146,6 +147,122 @@ def _cpu_attention_baselines() -> dict:
         "value": flops(8, 8, 128, 64, 4) / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
         "sample": f"the whole workload in fp32, per-direction SDPA + autograd, median of 5 runs, {dt * 1e3:.1f} ms",
     }
+    return out
+
+
+def _end_to_end_step(steps: int, with_cpu_baseline: bool) -> dict:
+    """One LBI scan backward step at the end-to-end configuration, run as the training loop runs it (reference
+    train/runners.py:361-372): 12 layers of d_model 768 (12 heads of 64), vocabulary 50257, 6 regions of 2 layers,
+    interface width 64, batch 8, sequence 1024, bf16 weights and activations, fp32 interface.  The forward (the
+    stand-in model of the test suite; the reference's own model in a deployment) runs outside the timed region;
+    timed is ``ScanADEngine.backward``: readout VJP, state Jacobians of the five regions the scan reads (region
+    input pullback, 64 directions), interface scan with its cross-check, parameter VJPs of all six regions, canvas
+    VJP - every region-level product on the HIP kernels.  Checked against dense fp32 ``loss.backward()`` of the same
+    rounded weights on the device; the host baseline is that dense backward in fp32 on the host threads."""
+    import copy
+
+    import torch
+
+    from latent_bounded_interfaces_amd import benchmarks as lbi_bench
+    from latent_bounded_interfaces_amd.backends import HipTransformerLowering
+    from latent_bounded_interfaces_amd.backward import ScanADEngine
+    from latent_bounded_interfaces_amd.backward.suffix_scan import propagate_state_adjoint_from_last_region_input
+    from oracle import lbi_model as olbi
+
+    device = torch.device("cuda", 0)
+    cfg = olbi.END_TO_END
+    batch, seq_len = olbi.END_TO_END_BATCH, olbi.END_TO_END_SEQ
+    cpu_model = olbi.end_to_end_model()
+    ids, targets = olbi.end_to_end_batch()
+    model = copy.deepcopy(cpu_model).to(device)
+    model.region_backend.lowering = HipTransformerLowering()
+    ids_d, targets_d = ids.to(device), targets.to(device)
+    engine = ScanADEngine(state_jacobian_mode="structured", local_vjp_mode="structured")
+
+    def forward():
+        logits, cache = model.forward_with_cache(ids_d)
+        return olbi.token_loss(logits, targets_d), cache
+
+    def timed(fn, count):
+        out = []
+        for _ in range(count):
+            loss, cache = forward()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            result = fn(loss, cache)
+            torch.cuda.synchronize()
+            out.append((time.perf_counter() - t0) * 1e3)
+            del loss, cache
+        return out, result
+
+    step = lambda loss, cache: engine.backward(model=model, loss=loss, cache=cache)
+    timed(step, 1)                                                    # warm-up (allocator, verify-once probe)
+    step_ms, result = timed(step, steps)
+    jac = lambda loss, cache: engine.pullback_provider.materialize_state_jacobian_t(model=model, cache=cache,
+                                                                                     skip_last=True)
+    jac_ms, jts = timed(jac, max(2, steps // 2))
+    g_last = torch.randn(batch, cfg["interface_width"], device=device)
+    scan_ms = _time_events(lambda: propagate_state_adjoint_from_last_region_input(
+        jts, g_last, num_regions=len(jts), materialize_suffix=True), 10, 2)
+
+    # error against the dense fp32 path on the device
+    dense_model = copy.deepcopy(model).float()
+    dense_model.region_backend.lowering = None
+    _, dense = olbi.dense_gradients(dense_model, ids_d, targets_d)
+    del dense_model
+    err = norm = 0.0
+    for name, want in dense.items():
+        if want is not None:
+            got = result.grad_map[name].double()
+            err += float(((got - want.double()) ** 2).sum())
+            norm += float((want.double() ** 2).sum())
+    del dense
+    torch.cuda.empty_cache()
+
+    # algorithmic work: region pullbacks with 64 directions (5 regions), one-direction sweeps with the weight
+    # gradients (as many flops again as the cotangent products) for all 6 regions, readout products (logits
+    # cotangent times the head weight, and its weight gradient)
+    shape = dict(dim=cfg["dim"], n_heads=cfg["n_heads"], n_kv_heads=cfg["n_kv_heads"],
+                 head_dim=cfg["dim"] // cfg["n_heads"], hidden=cfg["hidden"], layers=cfg["layers_per_region"],
+                 batch=batch, seq_len=seq_len)
+    regions = cfg["layers"] // cfg["layers_per_region"]
+    jac_flops = (regions - 1) * lbi_bench.region_flops(basis=cfg["interface_width"], **shape)["total"]
+    one = lbi_bench.region_flops(basis=1, **shape)
+    vjp_flops = regions * (2 * one["gemm"] + one["attention"])
+    head_flops = 2 * 2.0 * batch * seq_len * cfg["dim"] * cfg["vocab_size"]
+    flops = jac_flops + vjp_flops + head_flops
+    step_avg = statistics.fmean(step_ms)
+    tflops = flops / (step_avg * 1e-3) / 1e12
+    out = {
+        "workload": "LBI scan backward step as the training loop runs it (ScanADEngine.backward on a real forward "
+                    "cache): 12 layers d_model 768, 12 heads x 64, hidden 3072, conv 4, vocab 50257, 6 regions x 2 "
+                    "layers, interface width 64, B=8 T=1024, bf16 weights and activations, fp32 interface; forward "
+                    "outside the timed region",
+        "step_ms_avg": step_avg, "step_ms_min": min(step_ms), "steps_per_s": 1e3 / step_avg,
+        "tokens_per_s": batch * seq_len * 1e3 / step_avg,
+        "state_jacobians_ms": statistics.fmean(jac_ms), "interface_scan_ms": statistics.fmean(scan_ms),
+        "readout_local_vjps_canvas_ms": step_avg - statistics.fmean(jac_ms) - statistics.fmean(scan_ms),
+        "interface_scan_rms": result.diagnostics["interface_scan_rms"],
+        "relative_l2_error_vs_dense_fp32": (err / norm) ** 0.5,
+        "algorithmic_flops": {"state_jacobians": jac_flops, "local_vjps": vjp_flops, "readout": head_flops},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_MFMA_TFLOPS},
+    }
+    del model
+    torch.cuda.empty_cache()
+    if with_cpu_baseline:
+        # dense fp32 loss.backward() of the same model on the host threads, one of the eight sequences
+        host = cpu_model.float()
+        logits, _ = host.forward_with_cache(ids[:1])
+        loss = olbi.token_loss(logits, targets[:1])
+        t0 = time.perf_counter()
+        loss.backward()
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {
+            "value": 1.0 / (dt * batch), "unit": "steps/s", "cores": int(torch.get_num_threads()), "kind": "port",
+            "sample": f"dense fp32 loss.backward() of the same 12-layer model on 1 of the {batch} sequences "
+                      f"({dt:.2f} s wall), scaled by {batch}",
+        }
     return out
 
 
@@ -294,7 +411,7 @@ def main() -> int:
         torch.cuda.empty_cache()
         extra.update(lbi_bench.region_section(steps=max(3, args.steps // 4)))
         torch.cuda.empty_cache()
-        extra.update(lbi_bench.lbi_step_section(steps=3))
+        extra["lbi_backward_step_bf16_L12_D768_V50257_B8_T1024_d64"] = _end_to_end_step(3, not args.no_cpu_baseline)
         result["extra"] = extra
 
     if not args.no_cpu_baseline:
