@@ -6,7 +6,7 @@
 //   S^T  = K Q^T        A = K tile (LDS, shared), B = Q (registers)   lanes = queries, registers = keys
 //   P    = exp2(S^T c - lse2), once for the four directions
 //   dP^T = V dO_p^T     A = V tile (LDS, shared), B = dO_p (LDS, private to the wave)
-//   dS_p = P (dP_p - delta_p)
+//   dS_p = P (dP_p - delta_p)       delta_p = rowsum(dO_p o O), formed by this kernel and left for the dK/dV kernel
 //   dQ_p += dS_p K      A = dS_p (registers), B = K tile through transpose reads
 // K/V tiles of 32 keys arrive by global_load_lds into a two-stage ring (loop unrolled by
 // two, stage offsets are immediates); the wave's four d_out tiles are copied to LDS once.
@@ -17,15 +17,19 @@
 
 #include "lbi_attn_dkdv128.h"
 
+#ifndef LBI_DQ_GRING
+#define LBI_DQ_GRING 2
+#endif
+
 namespace lbi {
 namespace attn_mfma {
 
 template <typename T, int DH, int PB, bool CAUSAL>
 __global__ __launch_bounds__(256) void dq_ring_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                     const T* __restrict__ v, const T* __restrict__ d_out,
-                                                    const float* __restrict__ lse2, const float* __restrict__ delta,
-                                                    T* __restrict__ dq, int n_bh, int H, int P, int T_len,
-                                                    float scale) {
+                                                    const float* __restrict__ lse2, const float* __restrict__ o32,
+                                                    float* __restrict__ delta, T* __restrict__ dq, int n_bh, int H,
+                                                    int P, int T_len, float scale) {
     constexpr int KS = DH / 16, ND = DH / 32;
     constexpr int RB = DH * 2;               // bytes per tile row
     constexpr int CPR = DH / 8;              // 16-byte chunks per tile row
@@ -72,7 +76,10 @@ __global__ __launch_bounds__(256) void dq_ring_kernel(const T* __restrict__ q, c
         }
     };
 
-    // Resident: Q fragments (B operand of S^T), lse2 and delta of the lane's query.
+    // Resident: Q fragments (B operand of S^T), lse2 and delta of the lane's query.  delta_p[i] = sum_d
+    // d_out_p[i][d] O[i][d] is formed here, from the d_out tiles the wave has just put into LDS and the forward
+    // output row of the lane's query (two lanes per query, half the head dim each), and left in the workspace
+    // (negated) for the dK/dV kernel: every (direction, query) has exactly one owner wave.
     u32x4 qf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
@@ -84,13 +91,45 @@ __global__ __launch_bounds__(256) void dq_ring_kernel(const T* __restrict__ q, c
     for (int pp = 0; pp < PB; ++pp) {
         const int p = min(p0 + pp, P - 1);  // surplus slots redo the last direction; never stored
         const size_t row0 = (((size_t)b * P + p) * H + hh) * T_len + i0w;
-        my_delta[pp] = -delta[row0 + m];  // the workspace keeps -delta
 #pragma unroll
         for (int u = 0; u < CPR / 2; ++u) {
             const int slot = 64 * u + lane;
             const int r = slot / CPR, c = slot % CPR;
             const u32x4 val = *reinterpret_cast<const u32x4*>(d_out + (row0 + r) * DH + 8 * c);
             *reinterpret_cast<u32x4*>(gf_w + pp * TILE + tile_off<DH>(r, c)) = val;
+        }
+        my_delta[pp] = 0.0f;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the tiles are the wave's own: LDS runs in order
+    __builtin_amdgcn_wave_barrier();
+    {
+        const float* o_row = o32 + base + (size_t)(i0w + m) * DH + h * (DH / 2);
+#pragma unroll
+        for (int c = 0; c < CPR / 2; ++c) {
+            const f32x4 o_lo = *reinterpret_cast<const f32x4*>(o_row + 8 * c);
+            const f32x4 o_hi = *reinterpret_cast<const f32x4*>(o_row + 8 * c + 4);
+#pragma unroll
+            for (int pp = 0; pp < PB; ++pp) {
+                const u32x4 g4 = *reinterpret_cast<const u32x4*>(gf_w + pp * TILE + tile_off<DH>(m, h * (CPR / 2) + c));
+                float part = my_delta[pp];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    part = fmaf(Mma<T>::lo(g4[e]), o_lo[2 * e], part);
+                    part = fmaf(Mma<T>::hi(g4[e]), o_lo[2 * e + 1], part);
+                }
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    part = fmaf(Mma<T>::lo(g4[2 + e]), o_hi[2 * e], part);
+                    part = fmaf(Mma<T>::hi(g4[2 + e]), o_hi[2 * e + 1], part);
+                }
+                my_delta[pp] = part;
+            }
+        }
+#pragma unroll
+        for (int pp = 0; pp < PB; ++pp) {
+            my_delta[pp] += __shfl_xor(my_delta[pp], 32, 64);
+            if (active && h == 0 && p0 + pp < P)
+                delta[(((size_t)b * P + p0 + pp) * H + hh) * T_len + i0w + m] = -my_delta[pp];  // kept negated
         }
     }
 
@@ -132,8 +171,15 @@ __global__ __launch_bounds__(256) void dq_ring_kernel(const T* __restrict__ q, c
         u32x4 va[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) va[ks] = nat(vt, ks);
-        u32x4 gfr[2];  // d_out fragment ring
-        gfr[0] = nat(gf_w, 0);
+        // d_out fragment ring: fragment f = pp * KS + ks lives in slot f % GR and is fetched GR - 1 products ahead
+        // (an LDS read issued one product ahead arrives after that product has drained)
+        constexpr int GR = LBI_DQ_GRING;
+        u32x4 gfr[GR];
+        auto fetch_gf = [&](int f) __attribute__((always_inline)) {
+            if (f < PB * KS) gfr[f % GR] = nat(gf_w + (f / KS) * TILE, f % KS);
+        };
+#pragma unroll
+        for (int f = 0; f < GR - 1; ++f) fetch_gf(f);
         mma_v_settle(s);
 
         u32x4 pq[2];           // P rounded to the storage type
@@ -141,14 +187,11 @@ __global__ __launch_bounds__(256) void dq_ring_kernel(const T* __restrict__ q, c
         f32x16 dp_prev = s;    // placeholder until the first dP tile exists
 #pragma unroll
         for (int pp = 0; pp < PB; ++pp) {
-            const char* gt = gf_w + pp * TILE;
             f32x16 dp;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const int cur = (pp * KS + ks) & 1;
-                // next fragment: same direction, or the first one of the next direction
-                if (ks + 1 < KS) gfr[cur ^ 1] = nat(gt, ks + 1);
-                else if (pp + 1 < PB) gfr[cur ^ 1] = nat(gt + TILE, 0);
+                const int f = pp * KS + ks, cur = f % GR;
+                fetch_gf(f + GR - 1);
                 if (ks == 0) dp = Mma<T>::mma_v_start(va[0], gfr[cur]);
                 else Mma<T>::mma_v(va[ks], gfr[cur], dp);
                 // VALU work slotted under this product: P for pp == 0, dS_{pp-1} otherwise;
@@ -252,8 +295,8 @@ template <int DH, int PB> constexpr size_t dq_ring_lds_bytes() {
 // PB is the direction block of the caller's choice (1, 2, 4, and 8 for head dim 64); head dim 128 has
 // accumulation registers for four.
 template <typename T, int DH, int PB, bool CAUSAL>
-int launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
-               int H, int P, int T_len, float scale, hipStream_t stream) {
+int launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* o32, float* delta, T* dq,
+               int n_bh, int H, int P, int T_len, float scale, hipStream_t stream) {
     constexpr int PBK = (DH == 128 && PB > 4) ? 4 : PB;
     const int n_qb = (T_len + 127) / 128;
     const int n_pb = (P + PBK - 1) / PBK;
@@ -261,7 +304,7 @@ int launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2,
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");
     if (int rc = ensure_dynamic_lds<&dq_ring_kernel<T, DH, PBK, CAUSAL>>(lds_bytes)) return rc;
     hipLaunchKernelGGL((dq_ring_kernel<T, DH, PBK, CAUSAL>), dim3(grid_size(n_qb * n_pb, n_bh)), dim3(256), lds_bytes,
-                       stream, q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale);
+                       stream, q, k, v, g, lse2, o32, delta, dq, n_bh, H, P, T_len, scale);
     return LBI_OK;
 }
 

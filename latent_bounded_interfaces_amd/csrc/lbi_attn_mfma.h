@@ -2,12 +2,12 @@
 // T a multiple of 64, causal or not, fp32 accumulation.  (Short sequences run as one launch
 // instead: lbi_attn_small.h, built from the same fragments.)
 //
-// Four kernels per call, all atomic-free (every output tile has one owner, sums run
+// Three kernels per call, all atomic-free (every output tile has one owner, sums run
 // in a fixed order, so reruns are bit-identical):
 //   stats_kernel  flash-style forward: lse2[b,h,i] (log2 domain) and O = softmax(..) V (fp32)
-//   delta_kernel  -delta[b,p,h,i] = -sum_d d_out[b,p,h,i,d] * O[b,h,i,d]  (kept negated in the workspace)
 //   dq_ring_kernel    owner = 32 queries per wave, PB directions at once; streams K/V tiles
-//                     (lbi_attn_dq128.h)
+//                     (lbi_attn_dq128.h); it also forms -delta[b,p,h,i] = -sum_d d_out[b,p,h,i,d] * O[b,h,i,d]
+//                     from the d_out tiles it holds anyway and leaves it in the workspace
 //   dkdv_ring_kernel  owner = 64 keys per wave, one direction; streams Q/d_out tiles
 //                     (lbi_attn_dkdv128.h)
 //
@@ -319,43 +319,6 @@ __global__ __launch_bounds__(256) void stats_kernel(const T* __restrict__ q, con
     }
 }
 
-// ---------------------------------------------------------------------------------------
-// delta_kernel: DH/8 lanes per (b, h, t) row; a lane keeps its 32 bytes of O and walks the P
-// directions (16 bytes of d_out each), so O is read once and no index is divided per element.
-// ---------------------------------------------------------------------------------------
-template <typename T, int DH>
-__global__ __launch_bounds__(256) void delta_kernel(const T* __restrict__ d_out, const float* __restrict__ o32,
-                                                    float* __restrict__ delta, int H, int P, int T_len) {
-    constexpr int LPR = DH / 8;           // lanes per row
-    constexpr int ROWS = 256 / LPR;       // rows per workgroup
-    const int n_chunks = (T_len + ROWS - 1) / ROWS;
-    const int bh = blockIdx.x / n_chunks;  // b * H + h
-    const int t = (blockIdx.x - bh * n_chunks) * ROWS + threadIdx.x / LPR;
-    const int part = threadIdx.x % LPR;
-    const bool valid = t < T_len;
-    const int tc = valid ? t : T_len - 1;
-    const int b = bh / H, h = bh - b * H;
-    const float* o_ptr = o32 + ((size_t)bh * T_len + tc) * DH + part * 8;
-    const f32x4 o_lo = *reinterpret_cast<const f32x4*>(o_ptr);
-    const f32x4 o_hi = *reinterpret_cast<const f32x4*>(o_ptr + 4);
-    const size_t row0 = ((size_t)b * P * H + h) * T_len + tc;   // direction 0; + p * H * T_len
-    const size_t p_stride = (size_t)H * T_len;
-#pragma unroll 4
-    for (int p = 0; p < P; ++p) {
-        const size_t row = row0 + p * p_stride;
-        const u32x4 g = *reinterpret_cast<const u32x4*>(d_out + row * DH + part * 8);
-        const T* ge = reinterpret_cast<const T*>(&g);
-        float acc = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc = fmaf(to_f32(ge[e]), o_lo[e], acc);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc = fmaf(to_f32(ge[4 + e]), o_hi[e], acc);
-#pragma unroll
-        for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, LPR);
-        if (part == 0 && valid) delta[row] = -acc;  // stored negated: the dK/dV kernel starts dP from it
-    }
-}
-
 inline bool supports(int T_len, int dh, int dtype) {
     return (dtype == LBI_F16 || dtype == LBI_BF16) && (dh == 64 || dh == 128) && T_len >= 64 && T_len % 64 == 0;
 }
@@ -377,8 +340,8 @@ int launch_dkdv_pair(const T* q, const T* k, const T* v, const T* g, const float
 
 // dQ launch (kernel in lbi_attn_dq128.h); PB = directions per wave.
 template <typename T, int DH, int PB, bool CAUSAL>
-int launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* delta, T* dq, int n_bh,
-               int H, int P, int T_len, float scale, hipStream_t stream);
+int launch_dq(const T* q, const T* k, const T* v, const T* g, const float* lse2, const float* o32, float* delta, T* dq,
+               int n_bh, int H, int P, int T_len, float scale, hipStream_t stream);
 
 template <typename T, int DH, bool CAUSAL>
 int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T* dv, float* workspace, int B,
@@ -391,15 +354,13 @@ int launch_typed(const T* q, const T* k, const T* v, const T* g, T* dq, T* dk, T
     const int n_qb = (T_len + 127) / 128;
     hipLaunchKernelGGL((stats_kernel<T, DH, CAUSAL>), dim3(grid_size(n_qb, n_bh)), dim3(256), lds_bytes, stream, q, k,
                        v, lse2, o32, n_bh, T_len, scale);
-    constexpr int rows_per_block = 256 / (DH / 8);
-    hipLaunchKernelGGL((delta_kernel<T, DH>), dim3((unsigned)((T_len + rows_per_block - 1) / rows_per_block) * n_bh),
-                       dim3(256), 0, stream, g, o32, delta, H, P, T_len);
+    // the dQ kernel runs first: it writes -delta, which the dK/dV kernel reads
     // directions per wave of the dQ kernel: as many as share one S tile, without idle slots for one or two directions
     int rc;
-    if (P == 1) rc = launch_dq<T, DH, 1, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    else if (P == 2) rc = launch_dq<T, DH, 2, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    else if (DH == 64 && P > 4) rc = launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
-    else rc = launch_dq<T, DH, 4, CAUSAL>(q, k, v, g, lse2, delta, dq, n_bh, H, P, T_len, scale, stream);
+    if (P == 1) rc = launch_dq<T, DH, 1, CAUSAL>(q, k, v, g, lse2, o32, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else if (P == 2) rc = launch_dq<T, DH, 2, CAUSAL>(q, k, v, g, lse2, o32, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else if (DH == 64 && P > 4) rc = launch_dq<T, DH, 8, CAUSAL>(q, k, v, g, lse2, o32, delta, dq, n_bh, H, P, T_len, scale, stream);
+    else rc = launch_dq<T, DH, 4, CAUSAL>(q, k, v, g, lse2, o32, delta, dq, n_bh, H, P, T_len, scale, stream);
     if (rc) return rc;
     if (P >= 2) rc = launch_dkdv_pair<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
     else rc = launch_dkdv<T, DH, CAUSAL>(q, k, v, g, lse2, delta, dk, dv, n_bh, H, P, T_len, scale, stream);
