@@ -73,6 +73,29 @@ int lbi_suffix_scan_with_cotangents(const void* mats, const void* g, void* out, 
                                     int in_dtype, int out_dtype, void* stream);
 
 /*
+ * Both scan entries above with one more argument.  g and cot are both given (as lbi_suffix_scan_with_cotangents) or
+ * both null (as lbi_suffix_scan).  flags: 0, or LBI_SCAN_EXACT_SUFFIX.
+ *
+ * With bf16 storage at d = 256 the products run on the 16-bit matrix cores: the stored matrix enters as it is, the
+ * running suffix (fp32) as a sum of bf16 planes, accumulation is fp32.  By default the suffix operand is rounded to
+ * 16 significand bits (two planes: 256 times finer than the rounding of the stored inputs themselves; measured
+ * error against fp64 at K = 128 below 2e-4 of the largest entry, where the bar for 16-bit storage is 2e-2
+ * against the fp32 path); LBI_SCAN_EXACT_SUFFIX keeps its exact fp32 value (three planes, half again as many
+ * products): what is left is the rounding of the fp32 accumulation (measured <= 1.2e-5 at K = 128, <= 1e-5 on
+ * shorter chains).  The flag changes nothing for fp32 and fp16 storage or other
+ * widths, whose products are fp32 throughout.  The reference's native scan has one precision
+ * (cuda/interface/suffix_scan.cu:76-110: fp32 SGEMM, which its own tests allow TF32-sized errors,
+ * tests/test_interface_scan.py:34-39).
+ */
+enum lbi_scan_flags {
+    LBI_SCAN_EXACT_SUFFIX = 1
+};
+
+int lbi_suffix_scan_ex(const void* mats, const void* g, void* out, void* cot,
+                       int64_t B, int64_t K, int64_t d,
+                       int in_dtype, int out_dtype, int flags, void* stream);
+
+/*
  * Cotangent-only suffix chain: no d x d product is formed.
  *
  *   mats [B, K, d, d] (in_dtype), g [B, d] (fp32)  ->  out [B, K+1, d] (fp32)
@@ -144,8 +167,13 @@ int lbi_attn_pullback(const void* q, const void* k, const void* v, const void* d
  * are those of lbi_attn_pullback (the same kernels run, results are bit-identical).  A call whose
  * lbi_attn_pullback_workspace_bytes(...) exceeds LBI_ATTN_STATIC_SCRATCH_BYTES returns LBI_ERR_WORKSPACE.
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
- * threads) race on it; serialise them.  The first call on a device looks the array's address up
- * (hipGetSymbolAddress), later calls make no runtime call besides the launches.
+ * threads) race on it; serialise them.
+ *
+ * Runtime calls it makes: hipGetDevice on every call; on the FIRST call per device also hipGetSymbolAddress
+ * (the array's address on that device, kept afterwards) and, for kernels that need more than 64 KiB of LDS,
+ * hipFuncSetAttribute once per kernel and device.  None of these allocates, but the first-call ones must not
+ * happen for the first time inside a stream capture: make one call of the same shape outside the capture first
+ * (a warm-up), then capture; captured and later calls only launch kernels.
  */
 #define LBI_ATTN_STATIC_SCRATCH_BYTES (32u << 20)
 

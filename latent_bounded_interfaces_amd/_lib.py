@@ -15,7 +15,8 @@ LIB_PATH = Path(__file__).resolve().parent / "liblbi_hip.so"
 
 LBI_F32, LBI_F16, LBI_BF16 = 0, 1, 2
 ATTN_STATIC_SCRATCH_BYTES = 32 << 20  # LBI_ATTN_STATIC_SCRATCH_BYTES of include/lbi_hip.h
-ABI_VERSION = 8
+ABI_VERSION = 9
+LBI_SCAN_EXACT_SUFFIX = 1  # lbi_scan_flags of include/lbi_hip.h
 
 _DTYPE_CODES = {torch.float32: LBI_F32, torch.float16: LBI_F16, torch.bfloat16: LBI_BF16}
 
@@ -32,6 +33,11 @@ SYMBOLS = {
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_int,
          _c.c_void_p],
+    ),
+    "lbi_suffix_scan_ex": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_int,
+         _c.c_int, _c.c_void_p],
     ),
     "lbi_suffix_cotangents": (
         _c.c_int,

@@ -20,22 +20,26 @@ static __device__ __align__(256) unsigned char scratch[LBI_ATTN_STATIC_SCRATCH_B
 
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
-void* g_scratch_ptr[kMaxDevices] = {};
+std::atomic<void*> g_scratch_ptr[kMaxDevices];  // zero-initialised
 
-// Device address of `scratch` on the current device (looked up on the first call per device).
+// Device address of `scratch` on the current device.  Looked up on the first call per device (under a lock, with
+// hipGetSymbolAddress); every later call reads the kept pointer and makes no runtime call but hipGetDevice.
 int static_scratch(void** out) {
     int device = -1;
     LBI_HIP_CHECK(hipGetDevice(&device));
     if (device < 0 || device >= kMaxDevices)
         return fail(LBI_ERR_UNSUPPORTED, "lbi_attn_pullback_static: device index %d out of range", device);
-    std::lock_guard<std::mutex> guard(g_scratch_mutex);
-    if (!g_scratch_ptr[device]) {
-        void* ptr = nullptr;
-        LBI_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-        if (!ptr) return fail(LBI_ERR_HIP, "lbi_attn_pullback_static: scratch symbol has no device address");
-        g_scratch_ptr[device] = ptr;
+    void* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!ptr) {
+        std::lock_guard<std::mutex> guard(g_scratch_mutex);
+        ptr = g_scratch_ptr[device].load(std::memory_order_relaxed);
+        if (!ptr) {
+            LBI_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+            if (!ptr) return fail(LBI_ERR_HIP, "lbi_attn_pullback_static: scratch symbol has no device address");
+            g_scratch_ptr[device].store(ptr, std::memory_order_release);
+        }
     }
-    *out = g_scratch_ptr[device];
+    *out = ptr;
     return LBI_OK;
 }
 

@@ -22,6 +22,6 @@ void clear_error() { g_error[0] = '\0'; }
 
 }  // namespace lbi
 
-extern "C" int lbi_abi_version(void) { return 8; }
+extern "C" int lbi_abi_version(void) { return 9; }
 
 extern "C" const char* lbi_last_error(void) { return g_error; }

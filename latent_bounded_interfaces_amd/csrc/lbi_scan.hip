@@ -125,8 +125,8 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
     int r_top, r_lo = 0;
     bool write_tail = false;   // the start matrix and the identity behind it are results (out[K - 1], out[K])
     bool store_all = true;     // every step's product is a result
-    bool cot_on = COT;         // the cotangent chain of this workgroup is a result
-    bool cot_init = false;     // ... including its first vector (init_s @ g)
+    // the cotangent chain rides on the whole-chain form only; the chunk phases share no chain to carry it
+    static_assert(MODE == 0 || !COT, "chunk phases carry no cotangent chain");
     size_t stride_rt = DD;
     if constexpr (MODE == 0) {
         init_a = a_base + (size_t)(K - 1) * DD;
@@ -142,13 +142,11 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
             r_lo = c * plan.L;
             write_tail = last;
             store_all = last;
-            cot_on = COT && last;
         } else {
             const int c = seg;
             init_s = out_b + (size_t)(c + 1) * plan.L * DD;
             r_top = (c + 1) * plan.L - 1;
             r_lo = c == 0 ? 0 : c * plan.L + 1;   // out[cL] is a phase 2 result already
-            cot_init = c < plan.C - 2;            // out[(C-1)L] @ g is the last chunk's own chain value
         }
     } else if constexpr (MODE == 3) {
         const int c = seg + 1;
@@ -169,7 +167,6 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
         init_s = partner == plan.C - 1 ? out_b + (size_t)(plan.C - 1) * plan.L * DD
                                        : out_b + ((size_t)partner * plan.L + plan.rd) * DD;
         r_top = 0;
-        cot_on = false;
     } else {
         // step j multiplies the total parked in out[(j+1)L + 1] and stores out[(j+1)L]
         a_base = reinterpret_cast<const Tin*>(out_b + (size_t)(plan.L + 1) * DD);
@@ -177,7 +174,6 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
         stride_rt = (size_t)plan.L * DD;
         init_s = out_b + (size_t)(plan.C - 1) * plan.L * DD;
         r_top = plan.C - 3;
-        cot_on = false;
     }
     const bool from_a = MODE == 0 || (MODE == 1 && plan.phase == 1);  // start state: init_a, else init_s
     // distance between the matrices (and the results) of consecutive steps: a constant except in phase 2
@@ -235,11 +231,8 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 }
                 vbuf[row] = acc;
                 if (c0 == 0) {
-                    if (write_tail && cot_on) {
-                        cot_b[(size_t)K * D + row] = g_b[row];
-                        cot_b[(size_t)(K - 1) * D + row] = acc;
-                    }
-                    if (cot_init) cot_b[(size_t)(r_top + 1) * D + row] = acc;
+                    cot_b[(size_t)K * D + row] = g_b[row];
+                    cot_b[(size_t)(K - 1) * D + row] = acc;
                 }
             }
         }
@@ -371,7 +364,7 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
                 const float total = vdot[i] + __shfl_xor(vdot[i], 32, 64);  // the two k halves of a row
                 if (h == 0) {
                     v_new[row0 + i * 32 + m] = total;
-                    if (c0 == 0 && cot_on) cot_r[row0 + i * 32 + m] = total;
+                    if (c0 == 0) cot_r[row0 + i * 32 + m] = total;
                 }
             }
         }
@@ -887,7 +880,8 @@ constexpr int kWideBlockBatch = 512;
 // g / cot may be null (matrices only).  With them, the MFMA widths run the fused kernel;
 // other widths run the generic scan followed by the cotangent chain kernel.
 template <typename Tin>
-int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, int K, int d, hipStream_t stream) {
+int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, int K, int d, int flags,
+                hipStream_t stream) {
     // Few batch elements: one chain per column block leaves most of the chip idle for K - 1 dependent steps, so
     // the chain is cut into chunks that run side by side (ScanPlan), on narrow column blocks (short steps).
     ScanPlan plan{0, 0, 0, 0, 0, 0};
@@ -909,10 +903,11 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
     switch (d) {
         case 256: {
             // bf16 storage runs on the 16-bit matrix pipes: the running suffix enters each product as bf16
-            // planes (hi + mid + lo), the bf16 matrix as it is, accumulation in fp32.  Three planes (the default)
-            // are the fp32 value exactly.  LBI_SCAN_BF16_PLANES=2 rounds that operand to 16 significand bits,
-            // 256 times finer than the bf16 rounding of the inputs themselves (error against fp64 <= 2e-4 at
-            // K=128 where 2e-2 is asked of 16-bit storage), for two thirds of the products: 10-13 % faster.
+            // planes, the bf16 matrix as it is, accumulation in fp32.  Two planes (hi + mid, the default) round
+            // that operand to 16 significand bits, 256 times finer than the bf16 rounding of the inputs
+            // themselves (error against fp64 <= 2e-4 at K=128 where 2e-2 is asked of 16-bit storage), for two
+            // thirds of the products of the exact form; LBI_SCAN_EXACT_SUFFIX in `flags` asks for three planes
+            // (hi + mid + lo), which are the fp32 value exactly.
             // Matrices only: the column-owner kernel (a wave keeps its 16 columns of the suffix in registers, no
             // barrier between steps).  With the cotangent chain: the row-owner kernel, whose row dot products
             // carry the chain.  LBI_SCAN_ROW_OWNER=1 forces the latter.
@@ -921,7 +916,7 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
             // LBI_SCAN_SPLIT_FP32=1.
             if constexpr (std::is_same<Tin, bf16_raw>::value) {
                 static const bool row_owner = std::getenv("LBI_SCAN_ROW_OWNER") && std::atoi(std::getenv("LBI_SCAN_ROW_OWNER"));
-                static const int planes = std::getenv("LBI_SCAN_BF16_PLANES") ? std::atoi(std::getenv("LBI_SCAN_BF16_PLANES")) : 3;
+                const int planes = (flags & LBI_SCAN_EXACT_SUFFIX) ? 3 : 2;
                 if (!cot && !row_owner && K >= 1) return scan_col::launch(mats, out, B, K, planes, stream);
                 return scan_split::launch<Tin>(mats, out, g, cot, B, K, planes, stream);
             }
@@ -1038,11 +1033,16 @@ namespace lbi {
 namespace {
 
 int scan_entry(const char* what, const void* mats, void* out, const void* g, void* cot, int64_t B, int64_t K,
-               int64_t d, int in_dtype, int out_dtype, void* stream_v) {
+               int64_t d, int in_dtype, int out_dtype, int flags, void* stream_v) {
     clear_error();
+    if (flags & ~LBI_SCAN_EXACT_SUFFIX) return fail(LBI_ERR_INVALID, "%s: unknown flag bits 0x%x", what, flags);
     if (int rc = check_scan_args(what, mats, out, B, K, d, in_dtype)) return rc;
     if (out_dtype != LBI_F32) return fail(LBI_ERR_UNSUPPORTED, "%s: out_dtype must be LBI_F32", what);
     if (B == 0 || d == 0) return LBI_OK;
+    // widths that are a multiple of four run kernels with 16-byte accesses to every operand
+    if (d % 4 == 0 && (reinterpret_cast<uintptr_t>(mats) % 16 || reinterpret_cast<uintptr_t>(out) % 16 ||
+                       reinterpret_cast<uintptr_t>(g) % 16 || reinterpret_cast<uintptr_t>(cot) % 16))
+        return fail(LBI_ERR_INVALID, "%s: mats, out, g and cot must be 16-byte aligned", what);
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     if (K == 0) {
         const int64_t total = B * d * d;
@@ -1055,9 +1055,9 @@ int scan_entry(const char* what, const void* mats, void* out, const void* g, voi
         return LBI_OK;
     }
     switch (in_dtype) {
-        case LBI_F32: return launch_scan<float>(mats, out, g, cot, (int)B, (int)K, (int)d, stream);
-        case LBI_F16: return launch_scan<_Float16>(mats, out, g, cot, (int)B, (int)K, (int)d, stream);
-        default: return launch_scan<bf16_raw>(mats, out, g, cot, (int)B, (int)K, (int)d, stream);
+        case LBI_F32: return launch_scan<float>(mats, out, g, cot, (int)B, (int)K, (int)d, flags, stream);
+        case LBI_F16: return launch_scan<_Float16>(mats, out, g, cot, (int)B, (int)K, (int)d, flags, stream);
+        default: return launch_scan<bf16_raw>(mats, out, g, cot, (int)B, (int)K, (int)d, flags, stream);
     }
 }
 
@@ -1066,7 +1066,17 @@ int scan_entry(const char* what, const void* mats, void* out, const void* g, voi
 
 extern "C" int lbi_suffix_scan(const void* mats, void* out, int64_t B, int64_t K, int64_t d, int in_dtype,
                                int out_dtype, void* stream_v) {
-    return lbi::scan_entry("lbi_suffix_scan", mats, out, nullptr, nullptr, B, K, d, in_dtype, out_dtype, stream_v);
+    return lbi::scan_entry("lbi_suffix_scan", mats, out, nullptr, nullptr, B, K, d, in_dtype, out_dtype, 0, stream_v);
+}
+
+extern "C" int lbi_suffix_scan_ex(const void* mats, const void* g, void* out, void* cot, int64_t B, int64_t K,
+                                  int64_t d, int in_dtype, int out_dtype, int flags, void* stream_v) {
+    using namespace lbi;
+    if (B > 0 && d > 0 && ((g == nullptr) != (cot == nullptr))) {
+        clear_error();
+        return fail(LBI_ERR_INVALID, "lbi_suffix_scan_ex: g and cot must both be given or both be null");
+    }
+    return scan_entry("lbi_suffix_scan_ex", mats, out, g, cot, B, K, d, in_dtype, out_dtype, flags, stream_v);
 }
 
 extern "C" int lbi_suffix_scan_with_cotangents(const void* mats, const void* g, void* out, void* cot, int64_t B,
@@ -1076,7 +1086,7 @@ extern "C" int lbi_suffix_scan_with_cotangents(const void* mats, const void* g, 
         clear_error();
         return fail(LBI_ERR_INVALID, "lbi_suffix_scan_with_cotangents: g or cot is null");
     }
-    return scan_entry("lbi_suffix_scan_with_cotangents", mats, out, g, cot, B, K, d, in_dtype, out_dtype, stream_v);
+    return scan_entry("lbi_suffix_scan_with_cotangents", mats, out, g, cot, B, K, d, in_dtype, out_dtype, 0, stream_v);
 }
 
 extern "C" int lbi_suffix_cotangents(const void* mats, const void* g, void* out, int64_t B, int64_t K, int64_t d,

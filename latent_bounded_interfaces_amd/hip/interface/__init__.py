@@ -41,8 +41,13 @@ def _padded_width(rank: int) -> int:
     return next((w for w in _MFMA_WIDTHS if w > rank), rank)
 
 
-def suffix_scan_pullbacks(mats: torch.Tensor) -> torch.Tensor:
-    """``out[:, r] = mats[:, r] @ ... @ mats[:, K-1]``, ``out[:, K] = I``; fp32, input untouched."""
+def suffix_scan_pullbacks(mats: torch.Tensor, *, exact_suffix: bool = False) -> torch.Tensor:
+    """``out[:, r] = mats[:, r] @ ... @ mats[:, K-1]``, ``out[:, K] = I``; fp32, input untouched.
+
+    ``exact_suffix`` matters for bf16 storage at d = 256 only, whose products run on the 16-bit matrix cores with the
+    running suffix as a sum of bf16 planes: by default two planes (the suffix operand rounded to 16 significand bits,
+    error <= 2e-4 where 16-bit storage is asked 2e-2), with ``exact_suffix=True`` three (its exact fp32 value: only
+    the rounding of fp32 accumulation is left, ~1e-5 at K = 128; half again as many products)."""
     bsz, count, rank = _validate(mats)
     width = _padded_width(rank)
     if width != rank and mats.numel():
@@ -50,7 +55,7 @@ def suffix_scan_pullbacks(mats: torch.Tensor) -> torch.Tensor:
         # identity: run the matrix-core kernel of the next width instead of the scalar kernel (several times
         # faster even with the extra bytes).
         pad = width - rank
-        wide = suffix_scan_pullbacks(torch.nn.functional.pad(mats, (0, pad, 0, pad)))
+        wide = suffix_scan_pullbacks(torch.nn.functional.pad(mats, (0, pad, 0, pad)), exact_suffix=exact_suffix)
         return wide[:, :, :rank, :rank].contiguous()
     mats = mats.contiguous()
     out = torch.empty((bsz, count + 1, rank, rank), device=mats.device, dtype=torch.float32)
@@ -58,11 +63,11 @@ def suffix_scan_pullbacks(mats: torch.Tensor) -> torch.Tensor:
         return out
     lib = _lib.load()
     with torch.cuda.device(mats.device):
-        status = lib.lbi_suffix_scan(
-            mats.data_ptr(), out.data_ptr(), bsz, count, rank,
-            _lib.dtype_code(mats.dtype), _lib.LBI_F32, _lib.current_stream_ptr(mats.device),
+        status = lib.lbi_suffix_scan_ex(
+            mats.data_ptr(), None, out.data_ptr(), None, bsz, count, rank, _lib.dtype_code(mats.dtype), _lib.LBI_F32,
+            _lib.LBI_SCAN_EXACT_SUFFIX if exact_suffix else 0, _lib.current_stream_ptr(mats.device),
         )
-    _lib.check(status, "lbi_suffix_scan")
+    _lib.check(status, "lbi_suffix_scan_ex")
     return out
 
 
@@ -90,9 +95,11 @@ def suffix_scan_cotangents(mats: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor, *,
+                                         exact_suffix: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """Both results of the two functions above from one pass over ``mats`` (one kernel
-    for d in {32, 64, 128, 256}): ``(suffix [B, K+1, d, d], cotangents [B, K+1, d])``, fp32."""
+    for d in {32, 64, 128, 256}): ``(suffix [B, K+1, d, d], cotangents [B, K+1, d])``, fp32.
+    ``exact_suffix``: see :func:`suffix_scan_pullbacks`."""
     bsz, count, rank = _validate(mats)
     if g.dim() != 2 or g.shape[0] != bsz or g.shape[1] != rank:
         raise ValueError("g must have shape [B, R]")
@@ -100,7 +107,8 @@ def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor) ->
     if width != rank and mats.numel():
         pad = width - rank  # see suffix_scan_pullbacks; a zero-padded g leaves the first `rank` cotangents unchanged
         wide, wide_cot = suffix_scan_pullbacks_and_cotangents(torch.nn.functional.pad(mats, (0, pad, 0, pad)),
-                                                              torch.nn.functional.pad(g, (0, pad)))
+                                                              torch.nn.functional.pad(g, (0, pad)),
+                                                              exact_suffix=exact_suffix)
         return wide[:, :, :rank, :rank].contiguous(), wide_cot[:, :, :rank].contiguous()
     mats = mats.contiguous()
     g32 = g.to(device=mats.device, dtype=torch.float32).contiguous()
@@ -110,11 +118,12 @@ def suffix_scan_pullbacks_and_cotangents(mats: torch.Tensor, g: torch.Tensor) ->
         return out, cot
     lib = _lib.load()
     with torch.cuda.device(mats.device):
-        status = lib.lbi_suffix_scan_with_cotangents(
+        status = lib.lbi_suffix_scan_ex(
             mats.data_ptr(), g32.data_ptr(), out.data_ptr(), cot.data_ptr(), bsz, count, rank,
-            _lib.dtype_code(mats.dtype), _lib.LBI_F32, _lib.current_stream_ptr(mats.device),
+            _lib.dtype_code(mats.dtype), _lib.LBI_F32, _lib.LBI_SCAN_EXACT_SUFFIX if exact_suffix else 0,
+            _lib.current_stream_ptr(mats.device),
         )
-    _lib.check(status, "lbi_suffix_scan_with_cotangents")
+    _lib.check(status, "lbi_suffix_scan_ex")
     return out, cot
 
 

@@ -53,8 +53,8 @@ def suffix_scan_sequential(mats: torch.Tensor, dtype: torch.dtype | None = None)
     """
     bsz, count, rank = _check(mats)
     work = mats if dtype is None else mats.to(dtype)
-    out = torch.empty((bsz, count + 1, rank, rank), dtype=work.dtype)
-    run = torch.eye(rank, dtype=work.dtype).expand(bsz, rank, rank).clone()
+    out = torch.empty((bsz, count + 1, rank, rank), dtype=work.dtype, device=work.device)
+    run = torch.eye(rank, dtype=work.dtype, device=work.device).expand(bsz, rank, rank).clone()
     out[:, count] = run
     for r in range(count - 1, -1, -1):
         run = torch.matmul(work[:, r], run)

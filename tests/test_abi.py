@@ -48,6 +48,16 @@ def test_argument_validation_needs_no_gpu():
     assert lib.lbi_suffix_scan(None, None, 0, 2, 4, _lib.LBI_F32, _lib.LBI_F32, None) == 0
     assert lib.lbi_last_error() == b""
     assert lib.lbi_suffix_cotangents(None, None, None, 1, 2, 4, _lib.LBI_F32, None) == -1
+    # the scan entry with flags: unknown bits, g without cot, misaligned operands
+    ok = ctypes.c_void_p(256)
+    assert lib.lbi_suffix_scan_ex(ok, None, ok, None, 1, 2, 4, _lib.LBI_BF16, _lib.LBI_F32, 6, None) == -1
+    assert b"flag" in lib.lbi_last_error()
+    assert lib.lbi_suffix_scan_ex(ok, ok, ok, None, 1, 2, 4, _lib.LBI_BF16, _lib.LBI_F32, 0, None) == -1
+    assert b"both" in lib.lbi_last_error()
+    assert lib.lbi_suffix_scan_ex(ok, None, ctypes.c_void_p(260), None, 1, 2, 4, _lib.LBI_F32, _lib.LBI_F32,
+                                  _lib.LBI_SCAN_EXACT_SUFFIX, None) == -1
+    assert b"aligned" in lib.lbi_last_error()
+    assert lib.lbi_suffix_scan_ex(None, None, None, None, 0, 2, 4, _lib.LBI_F32, _lib.LBI_F32, 1, None) == 0
     assert lib.lbi_suffix_apply(None, None, None, 1, 2, 4, None) == -1
     assert b"null" in lib.lbi_last_error()
     assert lib.lbi_suffix_apply(None, None, None, -1, 2, 4, None) == -1

@@ -33,10 +33,12 @@ def _with_workspace(lib, q, k, v, g, scale, causal):
     return outs, need
 
 
-def _static(lib, q, k, v, g, scale, causal):
+def _static(lib, q, k, v, g, scale, causal, first_on_device=False):
     bsz, heads, seq, hd = q.shape
     outs = tuple(torch.full_like(g, float("nan")) for _ in range(3))
+    torch.cuda.synchronize()
     allocations = torch.cuda.memory_stats(q.device)["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info(q.device)[0]     # the driver's own count: sees a hipMalloc of the library too
     status = lib.lbi_attn_pullback_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(),
                                           *(o.data_ptr() for o in outs), bsz, heads, seq, hd, g.shape[1], scale,
                                           int(causal), _lib.dtype_code(q.dtype), _lib.current_stream_ptr(q.device))
@@ -44,6 +46,9 @@ def _static(lib, q, k, v, g, scale, causal):
     torch.cuda.synchronize()
     # nothing was taken from torch's allocator between entering and leaving the call
     assert torch.cuda.memory_stats(q.device)["allocation.all.allocated"] == allocations
+    if not first_on_device:
+        # (the first call on a device may make the runtime load the code object that holds the array)
+        assert torch.cuda.mem_get_info(q.device)[0] == free_before
     return outs
 
 
@@ -64,7 +69,7 @@ def test_static_scratch_entry_matches_the_workspace_entry(first, second, device)
             scale = shape[-1] ** -0.5
             want, need = _with_workspace(lib, q, k, v, g, scale, causal)
             assert 0 < need <= _lib.ATTN_STATIC_SCRATCH_BYTES      # the scratch array is really used
-            got = _static(lib, q, k, v, g, scale, causal)
+            got = _static(lib, q, k, v, g, scale, causal, first_on_device=index == 0)
             for name, a, b in zip(("dq", "dk", "dv"), got, want):
                 assert torch.equal(a, b), (name, index, shape)
 
@@ -88,3 +93,39 @@ def test_static_scratch_entry_python_wrapper_and_limit(device):
     with pytest.raises(RuntimeError, match="contiguous"):
         attention_input_pullback_basis_static(q.transpose(1, 2).contiguous().transpose(1, 2), k, v, g, out,
                                               softmax_scale=0.125)
+
+
+def test_static_scratch_entry_under_stream_capture(device):
+    """What the entry is for: after one warm-up call outside the capture (which does the per-device look-ups), a
+    call is captured into a graph and replayed; every replay, with eager work of the same entry in between, gives
+    the eager result bit for bit."""
+    lib = _lib.load()
+    q, k, v, g = _inputs((2, 4, 320, 64), 5, torch.float16, 91, device)
+    q2, k2, v2, g2 = _inputs((2, 4, 320, 64), 5, torch.float16, 92, device)
+    scale = 0.125
+    want, _ = _with_workspace(lib, q, k, v, g, scale, True)
+    want2, _ = _with_workspace(lib, q2, k2, v2, g2, scale, True)
+    outs = tuple(torch.zeros_like(g) for _ in range(3))
+    other = tuple(torch.zeros_like(g) for _ in range(3))
+
+    def call(args, dst):
+        a, b, c, d = args
+        status = lib.lbi_attn_pullback_static(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(),
+                                              *(o.data_ptr() for o in dst), 2, 4, 320, 64, 5, scale, 1,
+                                              _lib.dtype_code(a.dtype), _lib.current_stream_ptr(a.device))
+        _lib.check(status, "lbi_attn_pullback_static")
+
+    call((q, k, v, g), outs)                       # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call((q, k, v, g), outs)
+    for replay in range(3):
+        for o in outs:
+            o.zero_()
+        call((q2, k2, v2, g2), other)              # eager work on the same scratch array between replays
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(other, want2)), replay
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(outs, want)), replay
