@@ -45,6 +45,22 @@ int ensure_dynamic_lds(size_t bytes) {
     return LBI_OK;
 }
 
+// Compute units of the current device, asked of the runtime once per device and kept (256 on a whole MI355X, 32 per
+// partition when the part is split into its XCDs); 256 if the runtime will not say.  Launch plans that weigh "how
+// many workgroups fill the chip" use this figure.  The workgroup -> XCD dealing of the kernels (ids equal mod 8
+// share an L2) assumes the eight XCDs of an unpartitioned gfx950 part and is merely a permutation otherwise.
+inline int device_compute_units() {
+    constexpr int kTracked = 32;
+    static std::atomic<int> known[kTracked];  // zero-initialised
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kTracked) return 256;
+    int cus = known[dev].load(std::memory_order_relaxed);
+    if (cus > 0) return cus;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    known[dev].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));

@@ -808,7 +808,8 @@ int launch_mfma(const void* mats, void* out, const void* g, void* cot, int B, in
 
 // Chunking of the K-parallel scan: C chunks of L matrices.  The dependent depth is 2L + C - 3 steps, least at
 // L ~ sqrt(K / 2).  The chunked form does twice the products, which is free only while the plain form (B * nb
-// workgroups) leaves at least half of the 256 CUs idle; C is capped so that the widest phase stays within one
+// workgroups) leaves at least half of the CUs idle (256 on a whole MI355X; the count is asked of the runtime);
+// C is capped so that the widest phase stays within one
 // workgroup per CU, or within two where one would leave fewer than five chunks.  Measured at K = 128 (plain ->
 // chunked, ms per call): d = 256: B = 1: 2.36 -> 0.29, 4: 2.37 -> 0.37, 8: 2.04 -> 0.59, 16: 2.05 -> 1.14,
 // 32: 2.07 -> 2.3 (not taken); d = 128: B = 16: 0.35 -> 0.19, 48: 0.43 -> 0.57 (not taken).
@@ -818,9 +819,10 @@ inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
     if (forced == 0) return false;
     // chunks side by side: one workgroup per CU while that still leaves five or more of them (a step of two
     // workgroups sharing a CU takes 1.7x as long), else two per CU
-    const int one_per_cu = 256 / (B * nb) + 1;
-    const int cmax = one_per_cu >= 5 ? one_per_cu : 512 / (B * nb) + 1;
-    if (K < 12 || ((B * nb > 128 || cmax < 4) && forced <= 0)) return false;
+    const int cus = device_compute_units();
+    const int one_per_cu = cus / (B * nb) + 1;
+    const int cmax = one_per_cu >= 5 ? one_per_cu : 2 * cus / (B * nb) + 1;
+    if (K < 12 || ((B * nb > cus / 2 || cmax < 4) && forced <= 0)) return false;
     int L = 2;
     while (2 * (L + 1) * (L + 1) <= K) ++L;  // floor(sqrt(K / 2))
     if (forced > 0) L = forced < 2 ? 2 : forced;
@@ -874,8 +876,8 @@ int launch_chunked(const void* mats, void* out, const void* g, void* cot, int B,
 template <typename Tin>
 int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, int d, hipStream_t stream);
 
-// batch size from which one workgroup per batch element already fills the chip (two per CU)
-constexpr int kWideBlockBatch = 512;
+// batch size from which one workgroup per batch element already fills the chip (two per CU: 512 on a whole MI355X)
+inline int wide_block_batch() { return 2 * device_compute_units(); }
 
 // g / cot may be null (matrices only).  With them, the MFMA widths run the fused kernel;
 // other widths run the generic scan followed by the cotangent chain kernel.
@@ -929,7 +931,7 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
                 // Up to 32 batch elements the 64-wide blocks leave half the CUs or more without a workgroup: blocks
                 // of 32 columns (twice the workgroups, half the step time).
                 static const int narrow = std::getenv("LBI_SCAN_NARROW") ? std::atoi(std::getenv("LBI_SCAN_NARROW")) : -1;
-                if (narrow < 0 ? B <= 32 : narrow != 0) return launch_mfma<Tin, 256, 32, 32>(mats, out, g, cot, B, K, stream);
+                if (narrow < 0 ? B <= device_compute_units() / 8 : narrow != 0) return launch_mfma<Tin, 256, 32, 32>(mats, out, g, cot, B, K, stream);
             }
             return launch_mfma<Tin, 256, 32, 64>(mats, out, g, cot, B, K, stream);
         }
@@ -944,10 +946,10 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
             return cot ? launch_cotangent<Tin>(mats, g, cot, B, K, d, stream) : LBI_OK;
         }
         case 128:
-            if (B >= kWideBlockBatch) return launch_mfma<Tin, 128, 32, 128>(mats, out, g, cot, B, K, stream);
+            if (B >= wide_block_batch()) return launch_mfma<Tin, 128, 32, 128>(mats, out, g, cot, B, K, stream);
             return launch_mfma<Tin, 128, 32, 32>(mats, out, g, cot, B, K, stream);
         case 64:
-            if (B >= kWideBlockBatch) return launch_mfma<Tin, 64, 32, 64>(mats, out, g, cot, B, K, stream);
+            if (B >= wide_block_batch()) return launch_mfma<Tin, 64, 32, 64>(mats, out, g, cot, B, K, stream);
             return launch_mfma<Tin, 64, 32, 32>(mats, out, g, cot, B, K, stream);
         case 32: return launch_mfma<Tin, 32, 32, 32>(mats, out, g, cot, B, K, stream);
         default: break;
