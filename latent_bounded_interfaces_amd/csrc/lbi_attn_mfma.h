@@ -273,22 +273,31 @@ __global__ __launch_bounds__(256) void stats_kernel(const T* __restrict__ q, con
                 tmax = fmaxf(tmax, x);
             }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            // The reference point of the exponentials follows the running maximum only when that has grown by
+            // more than 2^8 (or is seen for the first time): the sums then carry terms of up to 2^8 instead of
+            // 1, which fp32 does not notice, and the rescaling of the 64 accumulator values of a lane, otherwise
+            // due on most steps, happens a few times per row.  O / l and m + log2 l do not depend on the choice.
             const float m_new = fmaxf(m_run, tmax);
-            const float alpha = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            const bool grow = (m_run == -INFINITY) ? (m_new != -INFINITY) : (m_new - m_run > 8.0f);
+            const float m_use = grow ? m_new : m_run;
             float lsum = 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float pr = (m_new == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(s[r] - m_new);
+                const float pr = (m_use == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(s[r] - m_use);
                 s[r] = pr;
                 lsum += pr;
             }
             lsum += __shfl_xor(lsum, 32, 64);
-            l_run = l_run * alpha + lsum;
-            m_run = m_new;
+            if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // wave-uniform
+                const float alpha = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_use);
+                l_run *= alpha;
 #pragma unroll
-            for (int nd = 0; nd < ND; ++nd)
+                for (int nd = 0; nd < ND; ++nd)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o_t[nd][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) o_t[nd][r] *= alpha;
+            }
+            l_run += lsum;
+            m_run = m_use;
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const u32x4 pb = pack_frag<T>(s, kk);

@@ -13,6 +13,7 @@
 #include "lbi_common.h"
 
 #include <cstdlib>
+#include <initializer_list>
 #include <type_traits>
 
 #include "lbi_scan_colsplit.h"
@@ -739,6 +740,205 @@ __global__ __launch_bounds__(512) void cotangent256_half_kernel(const Tin* __res
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// The d = 256 chain on FOUR workgroups per batch element, for batches that would otherwise leave three quarters
+// of the chip idle (a chain is one workgroup above, and a CU streams only ~50 GB/s on its own).  Workgroup `part`
+// of a group owns rows 64 part .. 64 part + 63 of every step's vector: eight streaming waves of eight rows each keep
+// their rows of the next matrices in flight (the same bytes in flight per CU as above, four matrices deep for fp32,
+// eight for 16-bit storage), and each step's 256-vector is exchanged through the result array itself: the owner
+// stores its 64 entries of out[b, r] (which are results anyway), the three partners pick them up from there.  The
+// array is filled with a marker word before the launch (a NaN payload no arithmetic produces; a result that
+// happened to equal it is stored as the canonical NaN instead), so a reader knows an entry has arrived when the
+// word differs from the marker: the data is its own flag, no ordering between two locations is relied on, and no
+// scratch memory is needed.  Stores and polls are agent-scope atomics (they bypass the non-coherent cache levels).
+//
+// The polls are made by a NINTH wave that does nothing else: loads return in order, so a streaming wave that
+// waited for a polled word would drain the matrix rows it has in flight on every step.
+//
+// Termination.  The four workgroups of a group have block ids that are equal mod 8 (one XCD, one L2) and the grid
+// is only launched when all of it is resident at once (4 B workgroups <= CUs).  A reader that has polled
+// `spin_limit` times without success stops waiting and computes the missing entry itself from the matrix row and
+// the vector it already holds, so every wave reaches every barrier whatever the partners do; the result is then
+// still correct to rounding (that entry is summed in another order than its owner's).
+// ---------------------------------------------------------------------------------------
+constexpr unsigned kChainMarker = 0x7fa5c3e1u;
+// polls (with a short sleep each) before a reader stops waiting for a partner: of the order of ten milliseconds
+constexpr int kChainSpinLimit = 1 << 14;
+
+__global__ __launch_bounds__(256) void fill_words_kernel(unsigned* __restrict__ p, size_t n, unsigned value) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        p[i] = value;
+}
+
+template <typename Tin>
+__global__ __launch_bounds__(576) void cotangent256_group_kernel(const Tin* __restrict__ mats,
+                                                                 const float* __restrict__ g, float* __restrict__ out,
+                                                                 int B, int K, int spin_limit) {
+    constexpr int D = 256, G = 4, ROWS = D / G, RPW = ROWS / 8;  // 64 rows per workgroup, 8 per streaming wave
+    constexpr bool WIDE = sizeof(Tin) == 4;
+    constexpr int RPL = WIDE ? 1 : 2;    // rows per load instruction (a 16-bit row is 512 bytes: one per lane half)
+    constexpr int LPM = RPW / RPL;       // load instructions per wave and matrix: 8 / 4
+    constexpr int DEPTH = 32 / LPM;      // matrices in flight: 4 / 8 (32 registers of 16 bytes either way)
+    constexpr int EPL = WIDE ? 4 : 8;    // elements per lane and load
+    typedef unsigned int raw4 __attribute__((ext_vector_type(4)));
+    __shared__ __align__(16) float vbuf[2][D];
+    const int id = blockIdx.x;
+    const int b = (id >> 5) * 8 + (id & 7);
+    const int part = (id >> 3) & 3;
+    if (b >= B) return;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int sub = WIDE ? 0 : lane >> 5, piece = WIDE ? lane : lane & 31;
+    const Tin* mats_b = mats + (size_t)b * K * D * D;
+    float* out_b = out + (size_t)b * (K + 1) * D;
+    const int row0 = part * ROWS;
+    if (tid < D) {
+        const float val = g[(size_t)b * D + tid];
+        vbuf[0][tid] = val;
+        if (tid >= row0 && tid < row0 + ROWS) out_b[(size_t)K * D + tid] = val;
+    }
+    if (K == 0) return;
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    if (wave == 8) {
+        // ---- the exchange wave: three foreign entries per lane and step
+        int idx[3];
+#pragma unroll
+        for (int e = 0; e < 3; ++e) {
+            const int f = lane + 64 * e;
+            idx[e] = f < row0 ? f : f + ROWS;
+        }
+        lds_barrier();
+        int cur = 0;
+        for (int r = K - 1; r >= 0; --r) {
+            unsigned* row_words = reinterpret_cast<unsigned*>(out_b + (size_t)r * D);
+            unsigned got[3] = {kChainMarker, kChainMarker, kChainMarker};
+            int spins = 0;
+            while (true) {
+                bool all = true;
+#pragma unroll
+                for (int e = 0; e < 3; ++e)
+                    if (got[e] == kChainMarker) {
+                        got[e] = __hip_atomic_load(row_words + idx[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        all = all && got[e] != kChainMarker;
+                    }
+                if (all) break;
+                if (++spins > spin_limit) {
+                    // the partner has not delivered: this entry from the matrix row and the vector at hand
+#pragma unroll
+                    for (int e = 0; e < 3; ++e)
+                        if (got[e] == kChainMarker) {
+                            const Tin* a_row = mats_b + (size_t)r * D * D + (size_t)idx[e] * D;
+                            float acc = 0.0f;
+                            for (int k = 0; k < D; k += 4) {
+                                const f32x4 a4 = load4(a_row + k);
+                                const f32x4 v4 = *reinterpret_cast<const f32x4*>(&vbuf[cur][k]);
+                                acc = fmaf(a4[3], v4[3], fmaf(a4[2], v4[2], fmaf(a4[1], v4[1], fmaf(a4[0], v4[0], acc))));
+                            }
+                            got[e] = __float_as_uint(acc);
+                        }
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+#pragma unroll
+            for (int e = 0; e < 3; ++e) vbuf[cur ^ 1][idx[e]] = __uint_as_float(got[e]);
+            lds_barrier();
+            cur ^= 1;
+        }
+        return;
+    }
+
+    // ---- streaming waves.  Load i of matrix r: row row0 + wave + 8 * (RPL * i + sub), elements EPL * piece ...
+    auto load_row = [&](int r, int i) {
+        return *reinterpret_cast<const raw4*>(mats_b + (size_t)r * D * D +
+                                              (size_t)(row0 + wave + 8 * (RPL * i + sub)) * D + EPL * piece);
+    };
+    raw4 buf[DEPTH][LPM];
+#pragma unroll
+    for (int s = 0; s < DEPTH; ++s)
+#pragma unroll
+        for (int i = 0; i < LPM; ++i) buf[s][i] = load_row(K - 1 - s > 0 ? K - 1 - s : 0, i);
+    lds_barrier();
+    int cur = 0;
+    auto step = [&](auto slot_tag, int r) __attribute__((always_inline)) {
+        constexpr int S = decltype(slot_tag)::value;
+        const f32x4 v_lo = *reinterpret_cast<const f32x4*>(&vbuf[cur][EPL * piece]);
+        f32x4 v_hi = v_lo;
+        if (!WIDE) v_hi = *reinterpret_cast<const f32x4*>(&vbuf[cur][EPL * piece + 4]);
+        const int r_fill = r - DEPTH > 0 ? r - DEPTH : 0;  // harmless re-reads at the end
+        float vals[LPM];
+#pragma unroll
+        for (int i = 0; i < LPM; ++i) {
+            if (WIDE) {
+                const raw4 w = buf[S][i];
+                vals[i] = fmaf(__uint_as_float(w[3]), v_lo[3],
+                               fmaf(__uint_as_float(w[2]), v_lo[2],
+                                    fmaf(__uint_as_float(w[1]), v_lo[1], __uint_as_float(w[0]) * v_lo[0])));
+            } else {
+                const Tin* e = reinterpret_cast<const Tin*>(&buf[S][i]);
+                float acc = to_f32(e[0]) * v_lo[0];
+#pragma unroll
+                for (int q = 1; q < 4; ++q) acc = fmaf(to_f32(e[q]), v_lo[q], acc);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc = fmaf(to_f32(e[4 + q]), v_hi[q], acc);
+                vals[i] = acc;
+            }
+            buf[S][i] = load_row(r_fill, i);
+            __builtin_amdgcn_sched_barrier(0);  // keep the refill next to the use
+        }
+        // halving butterfly over the lane bits 2 * HALF, then plain folds over the lane bits no value index uses
+        auto stage = [&](auto half_tag) {
+            constexpr int HALF = decltype(half_tag)::value;
+            const bool up = (lane & (2 * HALF)) != 0;
+            float got[HALF];
+#pragma unroll
+            for (int i = 0; i < HALF; ++i) got[i] = __shfl_xor(up ? vals[i] : vals[i + HALF], 2 * HALF, 64);
+#pragma unroll
+            for (int i = 0; i < HALF; ++i) vals[i] = (up ? vals[i + HALF] : vals[i]) + got[i];
+        };
+        if (WIDE) stage(std::integral_constant<int, 4>{});
+        stage(std::integral_constant<int, 2>{});
+        stage(std::integral_constant<int, 1>{});
+        float total = vals[0] + __shfl_xor(vals[0], 1, 64);
+        if (WIDE) {
+            total += __shfl_xor(total, 16, 64);
+            total += __shfl_xor(total, 32, 64);
+        } else {
+            total += __shfl_xor(total, 8, 64);
+            total += __shfl_xor(total, 16, 64);
+        }
+        const bool holder = WIDE ? (lane & 0x31) == 0 : (piece & 0x19) == 0;
+        if (holder) {
+            const int vi = WIDE ? (lane >> 1) & 7 : (piece >> 1) & 3;
+            const int row = row0 + wave + 8 * (RPL * vi + sub);
+            unsigned bits = __float_as_uint(total);
+            if (bits == kChainMarker) bits = 0x7fc00000u;
+            vbuf[cur ^ 1][row] = __uint_as_float(bits);
+            __hip_atomic_store(reinterpret_cast<unsigned*>(out_b + (size_t)r * D + row), bits, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        lds_barrier();
+        cur ^= 1;
+    };
+    auto steps = [&](int r_base, auto... slot_tags) __attribute__((always_inline)) {
+        // slots 0 .. DEPTH-1 hold matrices r_base, r_base - 1, ...; all waves leave together at the chain's end
+        (void)std::initializer_list<int>{(r_base - decltype(slot_tags)::value >= 0
+                                              ? (step(slot_tags, r_base - decltype(slot_tags)::value), 0)
+                                              : 0)...};
+    };
+    for (int r_base = K - 1; r_base >= 0; r_base -= DEPTH) {
+        if constexpr (DEPTH == 4)
+            steps(r_base, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{},
+                  std::integral_constant<int, 2>{}, std::integral_constant<int, 3>{});
+        else
+            steps(r_base, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{},
+                  std::integral_constant<int, 2>{}, std::integral_constant<int, 3>{},
+                  std::integral_constant<int, 4>{}, std::integral_constant<int, 5>{},
+                  std::integral_constant<int, 6>{}, std::integral_constant<int, 7>{});
+    }
+}
+
 // cot[b, r] = out[b, r] @ g[b] for M matrices per batch element: the cotangents of the K-parallel scan, whose
 // chunks have no common chain to carry them (M = K + 1; the identity tail gives cot[b, K] = g[b]), and the
 // entry point lbi_suffix_apply.  One workgroup per (b, r), a wave per row at a time, lanes along k (16-byte loads
@@ -975,6 +1175,24 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
     const size_t lds_bytes = (size_t)2 * dpad * sizeof(float);
     if (lds_bytes > 64 * 1024) return fail(LBI_ERR_UNSUPPORTED, "suffix cotangents: d=%d is too large (max 8192)", d);
     const int threads = d >= 128 ? 512 : (d >= 32 ? 256 : 64);
+    if (d == 256 && K >= 2 && 4 * B <= device_compute_units()) {
+        // few chains: four workgroups per chain, the vector exchanged through the result array (see the kernel)
+        // LBI_COT_GROUP=0 keeps one workgroup per chain; LBI_COT_SPIN_LIMIT sets the number of polls after which a
+        // reader stops waiting for its partners (0: never waits and forms every entry itself; for tests of that path)
+        static const int group = std::getenv("LBI_COT_GROUP") ? std::atoi(std::getenv("LBI_COT_GROUP")) : 1;
+        static const int spin_limit =
+            std::getenv("LBI_COT_SPIN_LIMIT") ? std::atoi(std::getenv("LBI_COT_SPIN_LIMIT")) : kChainSpinLimit;
+        if (group) {
+            const size_t words = (size_t)B * (K + 1) * d;
+            hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)((words + 1023) / 1024 > 1024 ? 1024 : (words + 1023) / 1024)),
+                               dim3(256), 0, stream, static_cast<unsigned*>(out), words, kChainMarker);
+            hipLaunchKernelGGL(cotangent256_group_kernel<Tin>, dim3((unsigned)((B + 7) / 8) * 32), dim3(576), 0, stream,
+                               static_cast<const Tin*>(mats), static_cast<const float*>(g), static_cast<float*>(out), B,
+                               K, spin_limit);
+            LBI_HIP_CHECK(hipGetLastError());
+            return LBI_OK;
+        }
+    }
     if (d == 256 && std::is_same<Tin, float>::value) {
         hipLaunchKernelGGL(cotangent256_kernel, dim3(B), dim3(512), 0, stream, static_cast<const float*>(mats),
                            static_cast<const float*>(g), static_cast<float*>(out), K);

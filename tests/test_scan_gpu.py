@@ -127,6 +127,48 @@ def test_cotangent_chain_matches_oracle(shape, dtype, device):
     assert torch.equal(got.cpu(), torch.tensor(case["cotangents"]))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bsz,count", [(1, 2), (3, 5), (13, 128), (64, 128), (64, 9), (65, 11)])
+def test_cotangent_chain_on_four_workgroups_per_element(bsz, count, dtype, device):
+    """d = 256 with at most a quarter as many chains as CUs: four workgroups share a chain and exchange each step's
+    vector through the result array (marker words).  Against the fp64 chain, terminal cotangent in place, no marker
+    left behind, reruns bit-identical; 65 chains take the one-workgroup kernel and must agree to rounding."""
+    from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents
+
+    mats, g = oscan.make_scan_inputs(bsz, count, 256, kind="near_identity", seed=21)
+    mats_d, g_d = mats.to(device).to(dtype), g.to(device)
+    out = suffix_scan_cotangents(mats_d, g_d)
+    assert torch.equal(out, suffix_scan_cotangents(mats_d, g_d)), "reruns differ"
+    assert bool(torch.isfinite(out).all()) and torch.equal(out[:, count], g_d)
+    truth = oscan.suffix_cotangents_sequential(mats_d.double().cpu(), g.double())
+    scale = truth.abs().amax(dim=2, keepdim=True).clamp_min(1e-30)
+    assert float(((out.cpu().double() - truth).abs() / scale).max()) <= 1e-5
+
+
+def test_cotangent_chain_partner_timeout_path_in_subprocess(device):
+    """A reader that gives up on its partners (forced from the host: LBI_COT_SPIN_LIMIT=0, no poll ever succeeds in
+    time) forms every missing entry itself: every wave still reaches every barrier and the chain is still right."""
+    import os
+    import subprocess
+    import sys
+
+    code = (
+        "import torch, sys; sys.path.insert(0, %r);"
+        "from oracle import scan as o;"
+        "from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents as f;"
+        "worst = 0.0\n"
+        "for dt in (torch.float32, torch.bfloat16):\n"
+        "    m, g = o.make_scan_inputs(5, 23, 256, kind='near_identity', seed=3); m = m.to(dt)\n"
+        "    out = f(m.cuda(), g.cuda()).cpu().double()\n"
+        "    t = o.suffix_cotangents_sequential(m.double(), g.double())\n"
+        "    worst = max(worst, float(((out - t).abs() / t.abs().amax(2, keepdim=True)).max()))\n"
+        "print(worst); sys.exit(0 if worst <= 1e-5 else 1)"
+    ) % str(Path(__file__).resolve().parents[1])
+    env = dict(os.environ, LBI_COT_SPIN_LIMIT="0")
+    res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stdout + res.stderr
+
+
 @pytest.mark.parametrize("shape", [(1, 0, 3), (2, 1, 8), (3, 5, 7), (4, 8, 32), (2, 6, 64), (3, 9, 128), (5, 12, 256),
                                    (9, 1, 256), (2, 2, 32), (2, 3, 100), (1, 1, 64), (2, 3, 512), (1, 2, 300)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
