@@ -761,9 +761,15 @@ __global__ __launch_bounds__(512) void cotangent256_half_kernel(const Tin* __res
 // the vector it already holds, so every wave reaches every barrier whatever the partners do; the result is then
 // still correct to rounding (that entry is summed in another order than its owner's).
 // ---------------------------------------------------------------------------------------
-constexpr unsigned kChainMarker = 0x7fa5c3e1u;
+using scan_col::kChainMarker;
 // polls (with a short sleep each) before a reader stops waiting for a partner: of the order of ten milliseconds
 constexpr int kChainSpinLimit = 1 << 14;
+// LBI_COT_SPIN_LIMIT overrides it (0: a reader never waits and forms every entry itself; for tests of that path)
+inline int chain_spin_limit() {
+    static const int limit =
+        std::getenv("LBI_COT_SPIN_LIMIT") ? std::atoi(std::getenv("LBI_COT_SPIN_LIMIT")) : kChainSpinLimit;
+    return limit;
+}
 
 __global__ __launch_bounds__(256) void fill_words_kernel(unsigned* __restrict__ p, size_t n, unsigned value) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
@@ -1120,6 +1126,16 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
                 static const bool row_owner = std::getenv("LBI_SCAN_ROW_OWNER") && std::atoi(std::getenv("LBI_SCAN_ROW_OWNER"));
                 const int planes = (flags & LBI_SCAN_EXACT_SUFFIX) ? 3 : 2;
                 if (!cot && !row_owner && K >= 1) return scan_col::launch(mats, out, B, K, planes, stream);
+                // With the chain, while all 4 B workgroups are resident at once: the same column-owner kernel with
+                // a fifth wave per workgroup that carries the chain (the four workgroups of a batch element
+                // exchange its vector through `cot`, which is filled with the marker word first).  Larger batches
+                // take the row-owner kernel, whose chain needs no exchange.
+                if (cot && !row_owner && K >= 1 && 4 * B <= device_compute_units()) {
+                    const size_t words = (size_t)B * (K + 1) * 256;
+                    hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)((words + 1023) / 1024)), dim3(256), 0, stream,
+                                       static_cast<unsigned*>(cot), words, kChainMarker);
+                    return scan_col::launch_with_chain(mats, out, g, cot, B, K, planes, chain_spin_limit(), stream);
+                }
                 return scan_split::launch<Tin>(mats, out, g, cot, B, K, planes, stream);
             }
             if constexpr (std::is_same<Tin, float>::value) {
@@ -1177,11 +1193,9 @@ int launch_cotangent(const void* mats, const void* g, void* out, int B, int K, i
     const int threads = d >= 128 ? 512 : (d >= 32 ? 256 : 64);
     if (d == 256 && K >= 2 && 4 * B <= device_compute_units()) {
         // few chains: four workgroups per chain, the vector exchanged through the result array (see the kernel)
-        // LBI_COT_GROUP=0 keeps one workgroup per chain; LBI_COT_SPIN_LIMIT sets the number of polls after which a
-        // reader stops waiting for its partners (0: never waits and forms every entry itself; for tests of that path)
+        // LBI_COT_GROUP=0 keeps one workgroup per chain
         static const int group = std::getenv("LBI_COT_GROUP") ? std::atoi(std::getenv("LBI_COT_GROUP")) : 1;
-        static const int spin_limit =
-            std::getenv("LBI_COT_SPIN_LIMIT") ? std::atoi(std::getenv("LBI_COT_SPIN_LIMIT")) : kChainSpinLimit;
+        const int spin_limit = chain_spin_limit();
         if (group) {
             const size_t words = (size_t)B * (K + 1) * d;
             hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)((words + 1023) / 1024 > 1024 ? 1024 : (words + 1023) / 1024)),

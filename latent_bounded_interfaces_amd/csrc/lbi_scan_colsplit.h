@@ -19,6 +19,17 @@
 // Per wave and step: 16 row tiles x 8 k-steps x 3 planes = 384 v_mfma_f32_16x16x32_bf16, 128 A-fragment
 // reads (one per three products), one fp32 accumulator per tile (the summation order of an fp32 dot
 // product with the three planes of a k-step taken small first).
+//
+// COT: the cotangent chain v_r = A_r v_{r+1} rides along on four more waves per workgroup (one per SIMD).  The four
+// workgroups of a batch element each own 64 entries of every v_r (workgroup = column block c <-> entries 64 c ..
+// 64 c + 63): four lanes of a chain wave share one row of A_r, read it from the chunks the matrix waves stream
+// through LDS anyway (no extra memory traffic) and sum 16 partial dot products of 16 terms in fp32.  The vector is exchanged between
+// the four workgroups through the result array cot[b, r, :] itself: it is filled with a marker word before the
+// launch, the owner stores its 64 entries, the others poll until the word differs from the marker (agent-scope
+// atomics; see cotangent256_group_kernel in lbi_scan.hip for the protocol and its bounded wait).  The entries of
+// v_{r+1} arrive some microseconds into step r, so the chain waves keep the chunks of their rows in registers and
+// multiply in the last quarter of the step, after one of them has picked the vector up.  The chain waves take part
+// in the chunk barriers and never wait for memory they do not expect to be there already.
 #pragma once
 
 #include "lbi_common.h"
@@ -73,9 +84,128 @@ __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c) {
 
 // NP = planes of the running suffix that enter the products: 3 is exact (the fp32 value), 2 rounds the operand to
 // 16 significand bits (hi + mid); the accumulation and the stored result are fp32 either way.
-template <int NP>
-__global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __restrict__ mats, float* __restrict__ out,
-                                                          int B, int K) {
+constexpr unsigned kChainMarker = 0x7fa5c3e1u;  // a NaN payload no arithmetic produces: "not written yet"
+
+// The chain waves of scan_colsplit_kernel<NP, true> (see the file comment): four per workgroup, one per SIMD, so that
+// their vector work spreads evenly under the matrix waves.  `part` = this workgroup's column block = its 64 entries
+// of the chain vector; chain wave cw owns rows 16 cw .. 16 cw + 15 of them, four lanes per row, a quarter of every
+// chunk's 64 k each (two 16-byte pieces).  They execute exactly the barriers of the matrix waves: four per step.
+__device__ __forceinline__ void chain_wave(const char* smem, float* vbuf, const bf16_raw* __restrict__ mats_b,
+                                           const float* __restrict__ g_b, float* __restrict__ cot_b, int part,
+                                           int cw, int lane, int K, int spin_limit) {
+    const int row = 64 * part + 16 * cw + (lane >> 2);   // this lane's row of every matrix, its entry of every vector
+    const int q = lane & 3;                              // its quarter of a chunk's k range
+    auto vb = [&](int r) { return vbuf + (r % 3) * D; };
+    auto chunk_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // one entry of A_r v_{r+1} straight from memory: the first vector, and the way out of a wait that ran out
+    auto entry_from_memory = [&](int r, int idx, const float* v) {
+        const bf16_raw* a_row = mats_b + (size_t)r * D * D + (size_t)idx * D;
+        float acc = 0.0f;
+        for (int k = 0; k < D; k += 4) {
+            const f32x4 a4 = load4(a_row + k);
+            const f32x4 v4 = *reinterpret_cast<const f32x4*>(v + k);
+            acc = fmaf(a4[3], v4[3], fmaf(a4[2], v4[2], fmaf(a4[1], v4[1], fmaf(a4[0], v4[0], acc))));
+        }
+        return acc;
+    };
+    auto publish = [&](int r, float value) {
+        unsigned bits = __float_as_uint(value);
+        if (bits == kChainMarker) bits = 0x7fc00000u;
+        vb(r)[row] = __uint_as_float(bits);
+        __hip_atomic_store(reinterpret_cast<unsigned*>(cot_b + (size_t)r * D + row), bits, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    };
+    // the 192 entries of v_r the partners own, three per lane of chain wave 0: polled until written (or formed here
+    // after `spin_limit` polls), then into the LDS copy
+    auto collect = [&](int r) {
+        unsigned* words = reinterpret_cast<unsigned*>(cot_b + (size_t)r * D);
+        int idx[3];
+        unsigned got[3] = {kChainMarker, kChainMarker, kChainMarker};
+#pragma unroll
+        for (int e = 0; e < 3; ++e) {
+            const int f = lane + 64 * e;
+            idx[e] = f < 64 * part ? f : f + 64;
+        }
+        int spins = 0;
+        while (true) {
+            bool all = true;
+#pragma unroll
+            for (int e = 0; e < 3; ++e)
+                if (got[e] == kChainMarker) {
+                    got[e] = __hip_atomic_load(words + idx[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    all = all && got[e] != kChainMarker;
+                }
+            if (all) break;
+            if (++spins > spin_limit) {
+#pragma unroll
+                for (int e = 0; e < 3; ++e)
+                    if (got[e] == kChainMarker) got[e] = __float_as_uint(entry_from_memory(r, idx[e], vb(r + 1)));
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+#pragma unroll
+        for (int e = 0; e < 3; ++e) vb(r)[idx[e]] = __uint_as_float(got[e]);
+    };
+    // the lane's two pieces (16 k) of chunk slot c; the pieces of a row are XOR-swizzled as the DMA laid them down
+    auto read_pieces = [&](u32x4 (&dst)[2], int c) {
+        const char* base = smem + c * CHUNK_BYTES + row * CHUNK_ROW_BYTES;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+            dst[t] = *reinterpret_cast<const u32x4*>(base + (((2 * q + t) ^ ((row >> 1) & 7)) << 4));
+    };
+    // 16 terms; v points at the lane's k range of the chunk
+    auto dot = [&](const u32x4 (&a)[2], const float* v) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const f32x4 lo = *reinterpret_cast<const f32x4*>(v + 8 * t);
+            const f32x4 hi = *reinterpret_cast<const f32x4*>(v + 8 * t + 4);
+            acc = fmaf(bf16_lo(a[t][0]), lo[0], acc);
+            acc = fmaf(bf16_hi(a[t][0]), lo[1], acc);
+            acc = fmaf(bf16_lo(a[t][1]), lo[2], acc);
+            acc = fmaf(bf16_hi(a[t][1]), lo[3], acc);
+            acc = fmaf(bf16_lo(a[t][2]), hi[0], acc);
+            acc = fmaf(bf16_hi(a[t][2]), hi[1], acc);
+            acc = fmaf(bf16_lo(a[t][3]), hi[2], acc);
+            acc = fmaf(bf16_hi(a[t][3]), hi[3], acc);
+        }
+        return acc;
+    };
+
+    // v_K = g (chain wave 0 keeps a copy and writes the owner's 64 entries of the result); v_{K-1} = A_{K-1} g, one
+    // lane per row, from memory
+    if (cw == 0) {
+        *reinterpret_cast<f32x4*>(vb(K) + 4 * lane) = *reinterpret_cast<const f32x4*>(g_b + 4 * lane);
+        cot_b[(size_t)K * D + 64 * part + lane] = g_b[64 * part + lane];
+    }
+    if (q == 0) publish(K - 1, entry_from_memory(K - 1, row, g_b));
+    for (int r = K - 2; r >= 0; --r) {
+        // The chunks of A_r pass through LDS one window each; v_{r+1} is complete in LDS only at the last barrier of
+        // the step (chain wave 0 picks the partners' entries up in the third window), so the pieces of the first
+        // three chunks wait in registers and all products are formed in the last window.
+        u32x4 piece[4][2];
+        chunk_barrier();
+        read_pieces(piece[0], 0);
+        chunk_barrier();
+        read_pieces(piece[1], 1);
+        chunk_barrier();
+        read_pieces(piece[2], 2);
+        if (cw == 0) collect(r + 1);                     // written by the partners at the end of the step before
+        chunk_barrier();
+        read_pieces(piece[3], 3);
+        const float* v = vb(r + 1) + 16 * q;
+        float acc = (dot(piece[0], v) + dot(piece[1], v + 64)) + (dot(piece[2], v + 128) + dot(piece[3], v + 192));
+        acc += __shfl_xor(acc, 1, 64);
+        acc += __shfl_xor(acc, 2, 64);
+        if (q == 0) publish(r, acc);
+    }
+}
+
+template <int NP, bool COT>
+__global__ __launch_bounds__(COT ? 2 * NT : NT) void scan_colsplit_kernel(
+    const bf16_raw* __restrict__ mats, float* __restrict__ out, const float* __restrict__ g_in,
+    float* __restrict__ cot, int B, int K, int spin_limit) {
     extern __shared__ __align__(16) char smem[];
     const int id = blockIdx.x;
     const int slot_id = id >> 3;
@@ -83,6 +213,12 @@ __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __res
     if (b >= B) return;
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    if (COT && wave >= NWAVE) {
+        chain_wave(smem, reinterpret_cast<float*>(smem + LDS_BYTES), mats + (size_t)b * K * D * D,
+                   g_in + (size_t)b * D, cot + (size_t)b * (K + 1) * D, slot_id % NB, wave - NWAVE, lane, K,
+                   spin_limit);
+        return;
+    }
     const int col = (slot_id % NB) * CB + wave * 16 + n;  // this lane's column of S
     const bf16_raw* mats_b = mats + (size_t)b * K * D * D;
     float* out_b = out + (size_t)b * (K + 1) * D * D;
@@ -224,19 +360,33 @@ __global__ __launch_bounds__(NT) void scan_colsplit_kernel(const bf16_raw* __res
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 }
 
-template <int NP>
-int launch_planes(const void* mats, void* out, int B, int K, hipStream_t stream) {
-    auto kern = scan_colsplit_kernel<NP>;
-    if (int rc = ensure_dynamic_lds<&scan_colsplit_kernel<NP>>(LDS_BYTES)) return rc;
+template <int NP, bool COT>
+int launch_planes(const void* mats, void* out, const void* g, void* cot, int B, int K, int spin_limit,
+                  hipStream_t stream) {
+    constexpr size_t lds_bytes = LDS_BYTES + (COT ? 3 * D * sizeof(float) : 0);   // + three copies of the chain vector
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");
+    auto kern = scan_colsplit_kernel<NP, COT>;
+    if (int rc = ensure_dynamic_lds<&scan_colsplit_kernel<NP, COT>>(lds_bytes)) return rc;
     const dim3 grid(((B + 7) / 8) * 8 * NB);
-    hipLaunchKernelGGL(kern, grid, dim3(NT), LDS_BYTES, stream, static_cast<const bf16_raw*>(mats),
-                       static_cast<float*>(out), B, K);
+    hipLaunchKernelGGL(kern, grid, dim3(COT ? 2 * NT : NT), lds_bytes, stream, static_cast<const bf16_raw*>(mats),
+                       static_cast<float*>(out), static_cast<const float*>(g), static_cast<float*>(cot), B, K,
+                       spin_limit);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
 
+// Matrices only.
 inline int launch(const void* mats, void* out, int B, int K, int planes, hipStream_t stream) {
-    return planes >= 3 ? launch_planes<3>(mats, out, B, K, stream) : launch_planes<2>(mats, out, B, K, stream);
+    return planes >= 3 ? launch_planes<3, false>(mats, out, nullptr, nullptr, B, K, 0, stream)
+                       : launch_planes<2, false>(mats, out, nullptr, nullptr, B, K, 0, stream);
+}
+
+// Matrices and the cotangent chain; `cot` must have been filled with kChainMarker on `stream` before.  Only for
+// batches whose 4 B workgroups are all resident at once (the chain waves of a batch element wait for each other).
+inline int launch_with_chain(const void* mats, void* out, const void* g, void* cot, int B, int K, int planes,
+                             int spin_limit, hipStream_t stream) {
+    return planes >= 3 ? launch_planes<3, true>(mats, out, g, cot, B, K, spin_limit, stream)
+                       : launch_planes<2, true>(mats, out, g, cot, B, K, spin_limit, stream);
 }
 
 }  // namespace scan_col

@@ -150,10 +150,19 @@ class OracleLBIModel(nn.Module):
         self.readout_norm = oreg.OracleRMSNorm(dim)
         self.lm_head = nn.Linear(dim, vocab_size, bias=False)
         with torch.no_grad():
+            # every parameter from the seeded generator (none from the process-wide one, whose state depends on
+            # what ran before): matrices ~ N(0, 1 / fan_in), biases ~ 0.1 N(0, 1), LayerNorm weights 1 + 0.1 N(0, 1);
+            # the update scale keeps its constant initial value
             for module in (self.canvas, self.interface, self.lm_head):
-                for p in module.parameters():
+                for name, p in module.named_parameters():
                     if p.dim() >= 2:
                         p.copy_(torch.randn(p.shape, generator=gen) * p.shape[-1] ** -0.5)
+                    elif name == "update_scale":
+                        continue
+                    elif "norms." in name and name.endswith("weight"):
+                        p.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=gen))
+                    else:
+                        p.copy_(0.1 * torch.randn(p.shape, generator=gen))
         self.canvas.to(dtype)
         self.readout_norm.to(dtype)
         self.lm_head.to(dtype)

@@ -64,7 +64,8 @@ def test_end_to_end_step_at_full_size_reproduces_dense_gradients(device):
         dot += float((got.double() * want.double()).sum())
         group = "interface" if name.startswith("interface") else \
             ("blocks" if name.startswith("region_backend") else name.split(".")[0])
-        by_group.setdefault(group, []).append(_relative_l2(got, want))
+        if want.numel() >= 64:      # a handful of scalars (the update scales) has no meaningful relative error
+            by_group.setdefault(group, []).append(_relative_l2(got, want))
     overall = (squared_error / squared_norm) ** 0.5
     cosine = dot / (got_norm ** 0.5 * squared_norm ** 0.5)
     worst = {group: max(values) for group, values in by_group.items()}

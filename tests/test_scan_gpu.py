@@ -147,7 +147,8 @@ def test_cotangent_chain_on_four_workgroups_per_element(bsz, count, dtype, devic
 
 def test_cotangent_chain_partner_timeout_path_in_subprocess(device):
     """A reader that gives up on its partners (forced from the host: LBI_COT_SPIN_LIMIT=0, no poll ever succeeds in
-    time) forms every missing entry itself: every wave still reaches every barrier and the chain is still right."""
+    time) forms every missing entry itself: every wave still reaches every barrier and the chain is still right, in
+    the cotangent-only kernel and in the chain waves of the fused bf16 scan."""
     import os
     import subprocess
     import sys
@@ -157,11 +158,18 @@ def test_cotangent_chain_partner_timeout_path_in_subprocess(device):
         "from oracle import scan as o;"
         "from latent_bounded_interfaces_amd.hip.interface import suffix_scan_cotangents as f;"
         "worst = 0.0\n"
+        "from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks_and_cotangents as fused\n"
         "for dt in (torch.float32, torch.bfloat16):\n"
         "    m, g = o.make_scan_inputs(5, 23, 256, kind='near_identity', seed=3); m = m.to(dt)\n"
         "    out = f(m.cuda(), g.cuda()).cpu().double()\n"
         "    t = o.suffix_cotangents_sequential(m.double(), g.double())\n"
         "    worst = max(worst, float(((out - t).abs() / t.abs().amax(2, keepdim=True)).max()))\n"
+        "m, g = o.make_scan_inputs(20, 7, 256, kind='near_identity', seed=4); m = m.to(torch.bfloat16)\n"
+        "mats, cot = fused(m.cuda(), g.cuda())\n"
+        "t = o.suffix_cotangents_sequential(m.double(), g.double())\n"
+        "worst = max(worst, float(((cot.cpu().double() - t).abs() / t.abs().amax(2, keepdim=True)).max()))\n"
+        "tm = o.suffix_scan_sequential(m.float(), dtype=torch.float64)\n"
+        "assert float(((mats.cpu().double() - tm).abs().flatten(2).amax(2) / tm.abs().flatten(2).amax(2)).max()) <= 2e-4\n"
         "print(worst); sys.exit(0 if worst <= 1e-5 else 1)"
     ) % str(Path(__file__).resolve().parents[1])
     env = dict(os.environ, LBI_COT_SPIN_LIMIT="0")
@@ -193,10 +201,12 @@ def test_fused_scan_and_cotangents(shape, dtype, device):
     assert float(((cot.cpu().double() - truth).abs() / scale).max()) <= 1e-5
 
 
-@pytest.mark.parametrize("shape", [(2, 5, 256), (9, 1, 256), (3, 12, 256), (2, 6, 64)])
+@pytest.mark.parametrize("shape", [(2, 5, 256), (9, 1, 256), (3, 12, 256), (2, 6, 64), (17, 9, 256), (64, 3, 256),
+                                   (65, 3, 256)])
 def test_fused_scan_and_cotangents_bf16_storage(shape, device):
-    """bf16 storage at d=256: the fused entry runs the row-owner split kernel (with the cotangent chain), the
-    matrices-only entry the column-owner one; with ``exact_suffix`` both are exact-split fp32 products in different
+    """bf16 storage at d=256: the matrices-only entry runs the column-owner kernel; the fused entry the same kernel
+    with chain waves (up to 64 batch elements: the four workgroups of an element exchange the chain vector) or the
+    row-owner split kernel (larger batches); with ``exact_suffix`` both are exact-split fp32 products in different
     summation orders, by default the suffix operand is rounded to 16 significand bits in both."""
     from latent_bounded_interfaces_amd.hip.interface import (
         suffix_scan_pullbacks,
