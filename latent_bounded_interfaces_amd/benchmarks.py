@@ -495,6 +495,8 @@ def main(argv=None) -> int:
     ap.add_argument("--out", default=None, help="--pmc-traffic: where to write the JSON (default: stdout)")
     ap.add_argument("--scan", nargs="*", default=None, help="time the fused suffix scan instead: B,K,d tuples")
     ap.add_argument("--matrices-only", action="store_true", help="--scan: the suffix matrices without the cotangents")
+    ap.add_argument("--cotangent-chain", nargs="*", default=None,
+                    help="time the cotangent-only chain (lbi_suffix_cotangents) instead: B,K,d tuples")
     args = ap.parse_args(argv)
     if args.pmc_traffic is not None:
         record = pmc_traffic(*args.pmc_traffic, kernel=args.kernel, copy_kernel=args.copy_kernel,
@@ -504,6 +506,12 @@ def main(argv=None) -> int:
             Path(args.out).write_text(text)
         else:
             sys.stdout.write(text)
+        return 0
+    if args.cotangent_chain is not None:
+        for spec in args.cotangent_chain:
+            B, K, d = (int(x) for x in spec.split(","))
+            print(json.dumps(measure_cotangent_chain(B, K, d, getattr(torch, args.dtype), warmup=args.warmup,
+                                                     iters=args.iters)), flush=True)
         return 0
     if args.scan is not None:
         for spec in args.scan:
