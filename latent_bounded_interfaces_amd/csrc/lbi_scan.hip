@@ -951,40 +951,68 @@ __global__ __launch_bounds__(576) void cotangent256_group_kernel(const Tin* __re
 // when d is a multiple of 4), butterfly fold.
 template <bool VEC4>
 __global__ __launch_bounds__(256) void suffix_apply_kernel(const float* __restrict__ out, const float* __restrict__ g,
-                                                           float* __restrict__ cot, int M, int d) {
-    const int b = blockIdx.x / M;
-    const float* mat = out + (size_t)blockIdx.x * d * d;
+                                                           float* __restrict__ cot, int M, int d, int rows_per_block,
+                                                           int parts) {
+    const int mat_id = blockIdx.x / parts;
+    const int row_begin = (blockIdx.x - mat_id * parts) * rows_per_block;
+    const int row_end = row_begin + rows_per_block < d ? row_begin + rows_per_block : d;
+    const int b = mat_id / M;
+    const float* mat = out + (size_t)mat_id * d * d;
     const float* g_b = g + (size_t)b * d;
-    float* cot_r = cot + (size_t)blockIdx.x * d;
+    float* cot_r = cot + (size_t)mat_id * d;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int row = wave; row < d; row += 4) {
-        float acc = 0.0f;
+    // four rows of a wave per trip, so that four loads per lane are in flight; each row's sum runs in the same
+    // order whatever the split
+    for (int row = row_begin + wave; row < row_end; row += 16) {
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         if (VEC4) {
             for (int k = lane * 4; k < d; k += 256) {
-                const f32x4 a4 = *reinterpret_cast<const f32x4*>(mat + (size_t)row * d + k);
                 const f32x4 v4 = *reinterpret_cast<const f32x4*>(g_b + k);
-                acc = fmaf(a4[0], v4[0], acc);
-                acc = fmaf(a4[1], v4[1], acc);
-                acc = fmaf(a4[2], v4[2], acc);
-                acc = fmaf(a4[3], v4[3], acc);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (row + 4 * u < row_end) {
+                        const f32x4 a4 = *reinterpret_cast<const f32x4*>(mat + (size_t)(row + 4 * u) * d + k);
+                        acc[u] = fmaf(a4[0], v4[0], acc[u]);
+                        acc[u] = fmaf(a4[1], v4[1], acc[u]);
+                        acc[u] = fmaf(a4[2], v4[2], acc[u]);
+                        acc[u] = fmaf(a4[3], v4[3], acc[u]);
+                    }
+                }
             }
         } else {
-            for (int k = lane; k < d; k += 64) acc = fmaf(mat[(size_t)row * d + k], g_b[k], acc);
+            for (int k = lane; k < d; k += 64) {
+                const float v = g_b[k];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (row + 4 * u < row_end) acc[u] = fmaf(mat[(size_t)(row + 4 * u) * d + k], v, acc[u]);
+            }
         }
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
-        if (lane == 0) cot_r[row] = acc;
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) acc[u] += __shfl_xor(acc[u], off, 64);
+            if (lane == 0 && row + 4 * u < row_end) cot_r[row + 4 * u] = acc[u];
+        }
     }
 }
 
 int launch_suffix_apply(const void* suffix, const void* g, void* cot, int64_t B, int64_t M, int d, hipStream_t stream) {
-    const dim3 grid((unsigned)(B * M));
+    // One workgroup per matrix when there are enough matrices to fill the chip several times over; with few of
+    // them (one batch element) a matrix is cut into row blocks of 64, 32 or 16 for as many workgroups.
+    int rows_per_block = d;
+    const int64_t want = 4 * (int64_t)device_compute_units();
+    for (int rpb : {64, 32, 16}) {
+        if (B * M * ((d + rows_per_block - 1) / rows_per_block) >= want) break;
+        if (rpb < d) rows_per_block = rpb;
+    }
+    const int parts = (d + rows_per_block - 1) / rows_per_block;
+    const dim3 grid((unsigned)(B * M * parts));
     if (d % 4 == 0)
         hipLaunchKernelGGL(suffix_apply_kernel<true>, grid, dim3(256), 0, stream, static_cast<const float*>(suffix),
-                           static_cast<const float*>(g), static_cast<float*>(cot), (int)M, d);
+                           static_cast<const float*>(g), static_cast<float*>(cot), (int)M, d, rows_per_block, parts);
     else
         hipLaunchKernelGGL(suffix_apply_kernel<false>, grid, dim3(256), 0, stream, static_cast<const float*>(suffix),
-                           static_cast<const float*>(g), static_cast<float*>(cot), (int)M, d);
+                           static_cast<const float*>(g), static_cast<float*>(cot), (int)M, d, rows_per_block, parts);
     LBI_HIP_CHECK(hipGetLastError());
     return LBI_OK;
 }
@@ -1012,31 +1040,56 @@ int launch_mfma(const void* mats, void* out, const void* g, void* cot, int B, in
                : launch_mfma_cot<Tin, D, RT, CB, false>(mats, out, nullptr, nullptr, B, K, stream);
 }
 
-// Chunking of the K-parallel scan: C chunks of L matrices.  The dependent depth is 2L + C - 3 steps, least at
-// L ~ sqrt(K / 2).  The chunked form does twice the products, which is free only while the plain form (B * nb
-// workgroups) leaves at least half of the CUs idle (256 on a whole MI355X; the count is asked of the runtime);
-// C is capped so that the widest phase stays within one
-// workgroup per CU, or within two where one would leave fewer than five chunks.  Measured at K = 128 (plain ->
-// chunked, ms per call): d = 256: B = 1: 2.36 -> 0.29, 4: 2.37 -> 0.37, 8: 2.04 -> 0.59, 16: 2.05 -> 1.14,
-// 32: 2.07 -> 2.3 (not taken); d = 128: B = 16: 0.35 -> 0.19, 48: 0.43 -> 0.57 (not taken).
+// Whether the products of the chunk totals (phase 2) run in log depth: level l multiplies every element by the one
+// 2^l places to its right, all chunks side by side, ceil(log2(C - 1)) launches of one step each, where the chain
+// takes C - 2 dependent steps.  The levels need the two slots of a chunk that phase 3 rewrites (L >= 3).
+inline int total_levels(int C) {
+    int levels = 0;
+    while ((1 << levels) < C - 1) ++levels;
+    return levels;
+}
+inline bool totals_in_log_depth(int L, int C) {
+    static const bool no_log = std::getenv("LBI_SCAN_TOTALS_CHAIN") && std::atoi(std::getenv("LBI_SCAN_TOTALS_CHAIN"));
+    return !no_log && L >= 3 && 2 * total_levels(C) <= C - 2;
+}
+
+// Chunking of the K-parallel scan: C chunks of L matrices.  The chunked form does twice the products, which is
+// free only while the plain form (B * nb workgroups) leaves at least half of the CUs idle (256 on a whole MI355X;
+// the count is asked of the runtime).  The dependent depth is 2L - 1 steps of the chunks plus the products of the
+// totals: C - 2 steps as a chain, or ceil(log2(C - 1)) launches of one step, each costing about 1.4 steps (12-13 us
+// against 9 us at d = 256).  L is the length with the least such depth among those whose chunks still fit two
+// workgroups per CU; where they need more than one per CU a step takes 1.7x as long.  Measured at K = 128, d = 256
+// (plain -> chunked, ms per call): B = 1: 2.36 -> 0.17 (L = 4; 0.21 at L = 8), 2: 2.36 -> 0.23, 4: 2.37 -> 0.35,
+// 8: 2.04 -> 0.59, 16: 2.05 -> 1.14, 32: 2.07 -> 2.3 (not taken); d = 128: B = 1: 0.070 at L = 4 (0.081 at L = 8),
+// 16: 0.35 -> 0.19, 48: 0.43 -> 0.57 (not taken).
 // Returns false when the plain chain is at least as good.  LBI_SCAN_CHUNK=0 forces the plain chain, n >= 2 chunks of n.
 inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
     static const int forced = std::getenv("LBI_SCAN_CHUNK") ? std::atoi(std::getenv("LBI_SCAN_CHUNK")) : -1;
-    if (forced == 0) return false;
-    // chunks side by side: one workgroup per CU while that still leaves five or more of them (a step of two
-    // workgroups sharing a CU takes 1.7x as long), else two per CU
-    const int cus = device_compute_units();
-    const int one_per_cu = cus / (B * nb) + 1;
-    const int cmax = one_per_cu >= 5 ? one_per_cu : 2 * cus / (B * nb) + 1;
-    if (K < 12 || ((B * nb > cus / 2 || cmax < 4) && forced <= 0)) return false;
-    int L = 2;
-    while (2 * (L + 1) * (L + 1) <= K) ++L;  // floor(sqrt(K / 2))
-    if (forced > 0) L = forced < 2 ? 2 : forced;
-    int C = (K + L - 1) / L;
-    if (C > cmax && forced <= 0) {
-        L = (K + cmax - 1) / cmax;
-        C = (K + L - 1) / L;
+    if (forced == 0 || K < 12) return false;
+    int L = 0;
+    if (forced > 0) {
+        L = forced < 2 ? 2 : forced;
+    } else {
+        const int cus = device_compute_units();
+        const int groups = B * nb;  // workgroups per chunk
+        if (groups > cus / 2) return false;
+        const int c_one = cus / groups + 1;      // C - 1 chunks side by side at one workgroup per CU
+        const int c_two = 2 * cus / groups + 1;  // at two
+        float best = 0.0f;
+        for (int cand = 2; (K + cand - 1) / cand >= 4; ++cand) {
+            const int C = (K + cand - 1) / cand;
+            if (C > c_two) continue;
+            float cost = (float)(2 * cand - 1) +
+                         (totals_in_log_depth(cand, C) ? 1.4f * (float)total_levels(C) : (float)(C - 2));
+            if (C > c_one) cost *= 1.7f;
+            if (L == 0 || cost <= best) {  // ties: the longer chunk (fewer launches)
+                best = cost;
+                L = cand;
+            }
+        }
+        if (L == 0) return false;
     }
+    const int C = (K + L - 1) / L;
     if (C < 4) return false;
     plan->L = L;
     plan->C = C;
@@ -1048,15 +1101,11 @@ inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
 template <typename Tin, int D, int RT, int CB>
 int launch_chunked(const void* mats, void* out, const void* g, void* cot, int B, int K, ScanPlan plan,
                    hipStream_t stream) {
-    // Phase 2 as a chain takes C - 2 dependent steps on B * D / CB workgroups.  With many chunks it runs in log
-    // depth instead: level l multiplies every element by the one 2^l places to its right, all chunks side by
-    // side, ceil(log2(C - 1)) launches of one step each.  The levels alternate between the two slots of a chunk
-    // that phase 3 rewrites anyway (out[cL + 1], where phase 1 parked the total, and out[cL + 2]: L >= 3) and the
-    // last one writes out[cL]; no slot is read and written in the same launch.
-    int levels = 0;
-    while ((1 << levels) < plan.C - 1) ++levels;
-    static const bool no_log = std::getenv("LBI_SCAN_TOTALS_CHAIN") && std::atoi(std::getenv("LBI_SCAN_TOTALS_CHAIN"));
-    const bool log_depth = !no_log && plan.L >= 3 && 2 * levels <= plan.C - 2;
+    // Phase 2 in log depth (totals_in_log_depth): the levels alternate between the two slots of a chunk that phase 3
+    // rewrites anyway (out[cL + 1], where phase 1 parked the total, and out[cL + 2]: L >= 3) and the last one writes
+    // out[cL]; no slot is read and written in the same launch.
+    const int levels = total_levels(plan.C);
+    const bool log_depth = totals_in_log_depth(plan.L, plan.C);
     for (int phase = 1; phase <= 3; ++phase) {
         plan.phase = phase;
         int rc = LBI_OK;
@@ -1117,8 +1166,8 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
             // thirds of the products of the exact form; LBI_SCAN_EXACT_SUFFIX in `flags` asks for three planes
             // (hi + mid + lo), which are the fp32 value exactly.
             // Matrices only: the column-owner kernel (a wave keeps its 16 columns of the suffix in registers, no
-            // barrier between steps).  With the cotangent chain: the row-owner kernel, whose row dot products
-            // carry the chain.  LBI_SCAN_ROW_OWNER=1 forces the latter.
+            // barrier between steps), with chain waves for the cotangents (below).  LBI_SCAN_ROW_OWNER=1 forces
+            // the row-owner kernel, whose row dot products carry the chain.
             // fp32 storage would need 3 x 3 planes: measured 4 % faster than the fp32-MFMA kernel and slightly
             // less accurate (the part clocks down under dense bf16 MFMA load), so it is opt-in:
             // LBI_SCAN_SPLIT_FP32=1.
@@ -1127,7 +1176,7 @@ int launch_scan(const void* mats, void* out, const void* g, void* cot, int B, in
                 const int planes = (flags & LBI_SCAN_EXACT_SUFFIX) ? 3 : 2;
                 if (!cot && !row_owner && K >= 1) return scan_col::launch(mats, out, B, K, planes, stream);
                 // With the chain, while all 4 B workgroups are resident at once: the same column-owner kernel with
-                // a fifth wave per workgroup that carries the chain (the four workgroups of a batch element
+                // four more waves per workgroup that carry the chain (the four workgroups of a batch element
                 // exchange its vector through `cot`, which is filled with the marker word first).  Larger batches
                 // take the row-owner kernel, whose chain needs no exchange.
                 if (cot && !row_owner && K >= 1 && 4 * B <= device_compute_units()) {

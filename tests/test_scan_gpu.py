@@ -353,7 +353,7 @@ def test_k_parallel_scan_long_chains(shape, device):
 
 @pytest.mark.parametrize("chunk,totals_chain", [(0, 0), (2, 0), (3, 0), (5, 0), (16, 0), (3, 1), (5, 1)])
 def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, totals_chain, device):
-    """LBI_SCAN_CHUNK forces the chunk length (0: the plain chain): every cut of K=13 / 33 / 64, including a
+    """LBI_SCAN_CHUNK forces the chunk length (0: the plain chain): every cut of K=13 / 29 / 33 / 64, including a
     one-matrix last chunk, meets the bar, with and without the cotangent chain.  The products of the chunk totals
     are formed in log depth where there are eight chunks or more and chunks of three matrices or more (chunk
     lengths 3 and 5 at K = 33 / 64 here; length 3 uses the last free slot of a chunk), as one chain otherwise;
@@ -368,7 +368,7 @@ def test_k_parallel_scan_forced_chunk_lengths_in_subprocess(chunk, totals_chain,
         "from latent_bounded_interfaces_amd.hip.interface import suffix_scan_pullbacks as s, "
         "suffix_scan_pullbacks_and_cotangents as f;"
         "worst = 0.0\n"
-        "for shape in ((1, 13, 64), (2, 33, 256), (1, 64, 32), (3, 21, 128)):\n"
+        "for shape in ((1, 13, 64), (2, 33, 256), (1, 64, 32), (3, 21, 128), (1, 29, 256)):\n"
         "    m, g = o.make_scan_inputs(*shape, kind='randn', seed=5)\n"
         "    t = o.suffix_scan_sequential(m, dtype=torch.float64)\n"
         "    c = o.suffix_cotangents_sequential(m.double(), g.double())\n"
