@@ -14,20 +14,22 @@ from torch import nn
 from .base import ADResult, GradMap, collect_named_grads
 
 
+def autograd_backward_step(model: nn.Module, *, ce_loss: torch.Tensor) -> GradMap:
+    """Named gradients of every trainable parameter from one dense backward of ``ce_loss``; gradients left on
+    the parameters from an earlier step are dropped first."""
+    for param in model.parameters():
+        param.grad = None
+    ce_loss.backward()
+    return collect_named_grads(model)
+
+
 class AutogradEngine:
-    """``backward(model=, loss=, cache=)`` clears the gradients, runs ``loss.backward()`` and returns the
-    named gradients; the cache is not read."""
+    """The dense step behind the engine interface (``backward(model=, loss=, cache=)``); the cache is not read."""
 
     name = "autograd"
 
     def backward(self, *, model: nn.Module, loss: torch.Tensor, cache: Any | None = None) -> ADResult:
-        model.zero_grad(set_to_none=True)
-        loss.backward()
-        return ADResult(grad_map=collect_named_grads(model))
-
-
-def autograd_backward_step(model: nn.Module, *, ce_loss: torch.Tensor) -> GradMap:
-    return AutogradEngine().backward(model=model, loss=ce_loss).grad_map
+        return ADResult(grad_map=autograd_backward_step(model, ce_loss=loss))
 
 
 __all__ = ["AutogradEngine", "autograd_backward_step"]
