@@ -47,8 +47,10 @@ SCAN_TRAFFIC_JSON = os.path.join(os.path.dirname(os.path.abspath(__file__)), "pr
 def _parse() -> argparse.Namespace:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20,
+                    help="untimed steps first: the part needs ~40 ms of load before its clock and the first-touch "
+                         "cost of the 2 GiB result settle")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline scan (used for profiling)")
     ap.add_argument("--cpu-sample-batch", type=int, default=64)
