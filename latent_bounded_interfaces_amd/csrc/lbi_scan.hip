@@ -49,25 +49,28 @@ namespace {
 // block 0 writes it.
 // Which part of the chain a workgroup runs.  `phase` 0 is the whole chain of a batch element (K - 1 dependent
 // steps).  Phases 1-3 are the K-parallel form for batches too small to fill the chip with one chain per column
-// block: the chain is cut into C chunks of L matrices and
+// block: the chain is cut into C chunks; chunk c >= 1 starts at matrix b_c = cL - s and has L matrices (the last
+// one what is left), chunk 0 has the first L - s (s = 1: every chunk then has L - 1 steps in phase 3, where chunk 0,
+// which has no boundary product of its own to skip, would otherwise run one step longer than the rest), and
 //   phase 1  every chunk c >= 1 multiplies its own matrices (L - 1 steps, all chunks side by side): the last chunk's
 //            products are final results and are stored as in phase 0; a middle chunk keeps only its total
-//            T_c = mats[cL] ... mats[(c+1)L - 1], parked in out[cL + 1], a slot phase 3 rewrites;
-//   phase 2  one chain over the totals (C - 2 steps): out[cL] = T_c @ out[(c+1)L] for c = C-2 ... 1, which are the
+//            T_c = mats[b_c] ... mats[b_c + L - 1], parked in out[b_c + 1], a slot phase 3 rewrites;
+//   phase 2  one chain over the totals (C - 2 steps): out[b_c] = T_c @ out[b_c + L] for c = C-2 ... 1, which are the
 //            final suffix products at the chunk boundaries (the kernel runs it with mats = the parked totals);
-//   phase 3  every chunk c <= C-2 restarts the chain from out[(c+1)L] through its own matrices (L - 1 or, for chunk
-//            0, L steps, all chunks side by side), storing each product.
+//   phase 3  every chunk c <= C-2 restarts the chain from out[b_{c+1}] through its own matrices (L - 1 steps, all
+//            chunks side by side), storing each product.
 // The cotangents, if asked for, are then the finished products applied to g (suffix_apply_kernel).
-// About twice the products, a dependent depth of 2L + C - 3 instead of K - 1, no scratch memory, no atomics; the
+// About twice the products, a dependent depth of 2L + C - 4 instead of K - 1, no scratch memory, no atomics; the
 // summation order is fixed by (K, L), so reruns are bit-identical.
 struct ScanPlan {
     int phase;  // 0: whole chain; 1, 2, 3: see above
     int L;      // matrices per chunk (>= 2)
     int C;      // chunks (>= 3)
-    // One level of the log-depth form of phase 2 (MODE 3): element c = 1 .. C-2 lives in slot out[cL + rd], the
-    // last element is out[(C-1)L]; the level writes elem[c] @ elem[c + off] (or elem[c] itself where c + off is
-    // past the last element) to out[cL + wr].
+    // One level of the log-depth form of phase 2 (MODE 3): element c = 1 .. C-2 lives in slot out[b_c + rd], the
+    // last element is out[b_{C-1}]; the level writes elem[c] @ elem[c + off] (or elem[c] itself where c + off is
+    // past the last element) to out[b_c + wr].
     int off, rd, wr;
+    int s;      // chunk boundaries b_c = cL - s (0 or 1)
 };
 
 // MODE 0: phase 0 only; every switch below is a compile-time constant, which keeps the whole-chain kernel at its
@@ -137,22 +140,22 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
         if (plan.phase == 1) {
             const int c = seg + 1;
             const bool last = c == plan.C - 1;
-            const int end = last ? K : (c + 1) * plan.L;
+            const int end = last ? K : (c + 1) * plan.L - plan.s;
             init_a = a_base + (size_t)(end - 1) * DD;
             r_top = end - 2;
-            r_lo = c * plan.L;
+            r_lo = c * plan.L - plan.s;
             write_tail = last;
             store_all = last;
         } else {
             const int c = seg;
-            init_s = out_b + (size_t)(c + 1) * plan.L * DD;
-            r_top = (c + 1) * plan.L - 1;
-            r_lo = c == 0 ? 0 : c * plan.L + 1;   // out[cL] is a phase 2 result already
+            init_s = out_b + (size_t)((c + 1) * plan.L - plan.s) * DD;
+            r_top = (c + 1) * plan.L - plan.s - 1;
+            r_lo = c == 0 ? 0 : c * plan.L - plan.s + 1;   // the chunk's first product is a phase 2 result already
         }
     } else if constexpr (MODE == 3) {
         const int c = seg + 1;
-        const float* left = out_b + ((size_t)c * plan.L + plan.rd) * DD;
-        float* dst = out_b + ((size_t)c * plan.L + plan.wr) * DD;
+        const float* left = out_b + (size_t)(c * plan.L - plan.s + plan.rd) * DD;
+        float* dst = out_b + (size_t)(c * plan.L - plan.s + plan.wr) * DD;
         const int partner = c + plan.off;
         if (partner > plan.C - 1) {
             // nothing to the right at this distance: the element is complete, it moves to the level's output slot
@@ -165,15 +168,15 @@ __global__ __launch_bounds__(64 * (D / RT)) void scan_mfma_kernel(
         }
         a_base = reinterpret_cast<const Tin*>(left);
         o_base = dst;
-        init_s = partner == plan.C - 1 ? out_b + (size_t)(plan.C - 1) * plan.L * DD
-                                       : out_b + ((size_t)partner * plan.L + plan.rd) * DD;
+        init_s = partner == plan.C - 1 ? out_b + (size_t)((plan.C - 1) * plan.L - plan.s) * DD
+                                       : out_b + (size_t)(partner * plan.L - plan.s + plan.rd) * DD;
         r_top = 0;
     } else {
-        // step j multiplies the total parked in out[(j+1)L + 1] and stores out[(j+1)L]
-        a_base = reinterpret_cast<const Tin*>(out_b + (size_t)(plan.L + 1) * DD);
-        o_base = out_b + (size_t)plan.L * DD;
+        // step j multiplies the total parked one slot above the first matrix of chunk j + 1 and stores that first slot
+        a_base = reinterpret_cast<const Tin*>(out_b + (size_t)(plan.L - plan.s + 1) * DD);
+        o_base = out_b + (size_t)(plan.L - plan.s) * DD;
         stride_rt = (size_t)plan.L * DD;
-        init_s = out_b + (size_t)(plan.C - 1) * plan.L * DD;
+        init_s = out_b + (size_t)((plan.C - 1) * plan.L - plan.s) * DD;
         r_top = plan.C - 3;
     }
     const bool from_a = MODE == 0 || (MODE == 1 && plan.phase == 1);  // start state: init_a, else init_s
@@ -947,8 +950,9 @@ __global__ __launch_bounds__(576) void cotangent256_group_kernel(const Tin* __re
 
 // cot[b, r] = out[b, r] @ g[b] for M matrices per batch element: the cotangents of the K-parallel scan, whose
 // chunks have no common chain to carry them (M = K + 1; the identity tail gives cot[b, K] = g[b]), and the
-// entry point lbi_suffix_apply.  One workgroup per (b, r), a wave per row at a time, lanes along k (16-byte loads
-// when d is a multiple of 4), butterfly fold.
+// entry point lbi_suffix_apply.  One workgroup per (b, r), or per block of rows of it when there are few matrices
+// (launch_suffix_apply); a wave takes four rows at a time, lanes along k (16-byte loads when d is a multiple of 4),
+// butterfly fold.
 template <bool VEC4>
 __global__ __launch_bounds__(256) void suffix_apply_kernel(const float* __restrict__ out, const float* __restrict__ g,
                                                            float* __restrict__ cot, int M, int d, int rows_per_block,
@@ -1055,7 +1059,7 @@ inline bool totals_in_log_depth(int L, int C) {
 
 // Chunking of the K-parallel scan: C chunks of L matrices.  The chunked form does twice the products, which is
 // free only while the plain form (B * nb workgroups) leaves at least half of the CUs idle (256 on a whole MI355X;
-// the count is asked of the runtime).  The dependent depth is 2L - 1 steps of the chunks plus the products of the
+// the count is asked of the runtime).  The dependent depth is 2L - 2 steps of the chunks plus the products of the
 // totals: C - 2 steps as a chain, or ceil(log2(C - 1)) launches of one step, each costing about 1.4 steps (12-13 us
 // against 9 us at d = 256).  L is the length with the least such depth among those whose chunks still fit two
 // workgroups per CU; where they need more than one per CU a step takes 1.7x as long.  Measured at K = 128, d = 256
@@ -1076,10 +1080,10 @@ inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
         const int c_one = cus / groups + 1;      // C - 1 chunks side by side at one workgroup per CU
         const int c_two = 2 * cus / groups + 1;  // at two
         float best = 0.0f;
-        for (int cand = 2; (K + cand - 1) / cand >= 4; ++cand) {
-            const int C = (K + cand - 1) / cand;
+        for (int cand = 2; (K + cand) / cand >= 4; ++cand) {
+            const int C = (K + cand) / cand;  // ceil((K + 1) / cand): boundaries at cL - 1
             if (C > c_two) continue;
-            float cost = (float)(2 * cand - 1) +
+            float cost = (float)(2 * cand - 2) +
                          (totals_in_log_depth(cand, C) ? 1.4f * (float)total_levels(C) : (float)(C - 2));
             if (C > c_one) cost *= 1.7f;
             if (L == 0 || cost <= best) {  // ties: the longer chunk (fewer launches)
@@ -1089,10 +1093,11 @@ inline bool plan_chunks(int B, int K, int nb, ScanPlan* plan) {
         }
         if (L == 0) return false;
     }
-    const int C = (K + L - 1) / L;
+    const int C = (K + L) / L;
     if (C < 4) return false;
     plan->L = L;
     plan->C = C;
+    plan->s = 1;
     return true;
 }
 
