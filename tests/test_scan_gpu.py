@@ -307,7 +307,10 @@ def test_k_parallel_scan_at_small_batches(bsz, kind, device):
 # chains long enough to be cut, at every matrix-core width the chunked form runs, lengths that leave a ragged or
 # one-matrix last chunk, batch sizes either side of the 8-chain launch mapping
 K_PARALLEL_SHAPES = [(1, 13, 32), (1, 37, 64), (2, 100, 128), (3, 61, 256), (1, 12, 256), (1, 129, 256), (9, 33, 32),
-                     (7, 50, 64), (2, 17, 100), (1, 40, 200)]
+                     (7, 50, 64), (2, 17, 100), (1, 40, 200),
+                     # chunk boundaries sit at cL - 1: lengths that make the last chunk one matrix, a full chunk, and
+                     # the shortest chains the planner cuts
+                     (1, 15, 256), (1, 16, 256), (2, 47, 256), (1, 255, 128), (4, 128, 32), (1, 14, 64)]
 
 
 @pytest.mark.parametrize("shape", K_PARALLEL_SHAPES)
