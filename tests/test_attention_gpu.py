@@ -88,10 +88,12 @@ LOWP_CASES = [
     # the same kernel at lengths that are no multiple of 32 (zero rows in the last tile, keys past the end masked)
     (37, (1, 2, 1, 64), 2), (38, (2, 1, 255, 64), 3), (39, (1, 2, 127, 128), 2), (40, (1, 1, 31, 64), 1),
     (41, (2, 2, 129, 64), 2), (42, (1, 1, 5, 128), 3),
-    # past the single-launch limits with direction counts that leave the four-kernel path a ragged tail: a last
-    # dQ group of fewer than 8 (Dh = 64) or 4 (Dh = 128) directions, an unpaired last direction in dK/dV
+    # past the single-launch limits with direction counts that leave the kernels a ragged tail: a last dQ group of
+    # fewer than 8 (Dh = 64) or 4 (Dh = 128) directions, a last dK/dV group of fewer than 4 (Dh = 64, two directions
+    # per wave) or an unpaired last direction (Dh = 128)
     (43, (1, 2, 320, 64), 5), (44, (1, 1, 320, 64), 9), (45, (1, 2, 192, 128), 3), (46, (1, 1, 320, 128), 5),
     (47, (1, 1, 384, 64), 11), (48, (2, 1, 192, 128), 7), (49, (1, 1, 512, 64), 3), (50, (1, 1, 256, 128), 9),
+    (51, (1, 2, 320, 64), 6), (52, (2, 1, 384, 64), 7), (53, (1, 3, 576, 64), 4), (54, (1, 1, 320, 64), 2),
 ]
 
 
