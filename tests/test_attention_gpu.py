@@ -184,6 +184,23 @@ def test_modes_and_contract(device):
         low.parameter_vjp(backend=None, cache=None, output_cotangent=torch.zeros(1, 2, 3, 4))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape,basis", [((2, 3, 384, 64), 11), ((1, 2, 320, 128), 7), ((1, 2, 1024, 64), 16)])
+def test_results_do_not_depend_on_how_directions_are_grouped(shape, basis, dtype, device):
+    """A direction's dQ, dK, dV are the same bits whether it is computed alone, in a pair, or among all directions:
+    the kernels group directions (eight or four per dQ workgroup, two per dK/dV workgroup, four at head dim 64 with
+    a second direction per wave) only to share the S / P tiles; every direction keeps its own products and sums."""
+    from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis
+
+    q, k, v, g = (t.to(device) for t in oattn.make_attention_inputs(*shape, basis, dtype=dtype, seed=77))
+    scale = 1.0 / math.sqrt(shape[-1])
+    whole = attention_input_pullback_basis(q, k, v, g, softmax_scale=scale, kernel_mode="hip")
+    for lo, hi in ((0, 2), (2, 3), (3, 6), (basis - 4, basis), (basis - 1, basis)):
+        part = attention_input_pullback_basis(q, k, v, g[:, lo:hi].contiguous(), softmax_scale=scale, kernel_mode="hip")
+        for name, a, b in zip(("dq", "dk", "dv"), part, whole):
+            assert torch.equal(a, b[:, lo:hi]), (name, lo, hi)
+
+
 def test_long_context_properties(device):
     """bf16, T=4096, Dh=128, P=16 on two (b, h) slices: size-independent checks."""
     from latent_bounded_interfaces_amd.hip.transformer import attention_input_pullback_basis
